@@ -1,0 +1,217 @@
+/*
+ * C-ABI of libpithtrain_hip.so: hand-written gfx950 kernels for PithTrain's FP8
+ * grouped-expert path.  Plain pointers and sizes only; every pointer is a device
+ * pointer unless it says "host".  All launches go to `stream` (a hipStream_t passed
+ * as void*); nothing here synchronises, allocates or frees device memory.
+ *
+ * Return value: 0 on success, negative PT_ERR_* otherwise; pt_last_error() gives a
+ * thread-local message for the last failure.
+ *
+ * Each entry point names the reference interface it replaces
+ * (paths relative to the PithTrain source tree).
+ */
+#ifndef PITHTRAIN_HIP_H
+#define PITHTRAIN_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* pt_stream_t;
+
+enum { PT_OK = 0, PT_ERR_INVALID = -1, PT_ERR_LAUNCH = -2, PT_ERR_UNSUPPORTED = -3 };
+/* element types of bf16/fp32/fp16 tensors */
+enum { PT_BF16 = 0, PT_F32 = 1, PT_F16 = 2 };
+
+const char* pt_last_error(void);
+int pt_abi_version(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Blockwise FP8 (e4m3fn) quantisation, power-of-two fp32 scales.
+ * Replaces pithtrain/operators/deepgemm_quantize.py (six Triton kernels).
+ * x is [M,N] with row stride ldx (elements) and unit column stride.
+ * ------------------------------------------------------------------------------------------ */
+
+/* layout of the colwise twin written by pt_quant_rowwise_colwise */
+enum {
+  PT_CH_ROWMAJOR = 0,  /* ch_fp8[M,N],  ch_scale[M/128,N]   fp8cast_rowwise_colwise :204-259 */
+  PT_CH_TRANSPOSED = 1,/* ch_fp8[N,M],  ch_scale[M/128,N]   (layout of this library's wgrad GEMM) */
+  PT_CH_KMAJOR = 2     /* flat per-group (N,K_g) blocks, ch_scale[N,M/128]  fp8cast_rowwise_kmajor :262-333 */
+};
+
+/* 1x128 rowwise + 128-row colwise from one read.  M % 128 == 0 (deepgemm_quantize.py:219).
+ * offs/num_groups are read only for PT_CH_KMAJOR (int32 inclusive row offsets, multiples of 128,
+ * offs[num_groups-1] == M). */
+int pt_quant_rowwise_colwise(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
+                             void* tok_fp8, float* tok_scale, void* ch_fp8, float* ch_scale,
+                             int ch_layout, const int32_t* offs, int32_t num_groups,
+                             pt_stream_t stream);
+
+/* rowwise(x) + rowwise(x^T): t_fp8[N,M], t_scale[N,ceil(M/128)].
+ * fp8cast_rowwise_transpose, deepgemm_quantize.py:429-482 */
+int pt_quant_rowwise_transpose(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
+                               void* tok_fp8, float* tok_scale, void* t_fp8, float* t_scale,
+                               pt_stream_t stream);
+
+/* rowwise(x) + 128x128 blockwise(x^T): blk_t_fp8[K,M], blk_t_scale[ceil(K/128),ceil(M/128)].
+ * fp8cast_rowwise_blockwise_transpose, deepgemm_quantize.py:575-629 */
+int pt_quant_rowwise_blockwise_transpose(const void* x, int dtype, int64_t M, int64_t K,
+                                         int64_t ldx, void* tok_fp8, float* tok_scale,
+                                         void* blk_t_fp8, float* blk_t_scale, pt_stream_t stream);
+
+/* 128x128 blockwise(x) + blockwise(x^T) for x[G,N,K] (element strides stride_g, stride_row):
+ * fp8[G,N,K], scale[G,ceil(N/128),ceil(K/128)], fp8_t[G,K,N], scale_t[G,ceil(K/128),ceil(N/128)].
+ * fp8cast_blockwise_transpose (:709-756, G == 1) and fp8cast_blockwise_transpose_batched
+ * (:846-899). */
+int pt_quant_blockwise_transpose_batched(const void* x, int dtype, int64_t G, int64_t N, int64_t K,
+                                         int64_t stride_g, int64_t stride_row, void* fp8,
+                                         float* scale, void* fp8_t, float* scale_t,
+                                         pt_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * FP8 GEMMs (fp32 accumulate on the MFMA units, scales applied in hardware as E8M0).
+ * Replace the DeepGEMM call sites of pithtrain/operators/linear.py and grouped_linear.py.
+ * ------------------------------------------------------------------------------------------ */
+
+/* out[m,n] = sum_k a[m,k] b[n,k];  a_scale[M,ceil(K/128)] (1x128), b_scale[ceil(N/128),ceil(K/128)]
+ * (128x128).  out is bf16 [M,N] (out_dtype PT_BF16) or fp32 (PT_F32).
+ * deep_gemm.fp8_fp4_gemm_nt at linear.py:40 (forward :57, dgrad :77, wgrad :80). */
+int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const void* b_fp8,
+                     const float* b_scale, void* out, int out_dtype, int64_t M, int64_t N,
+                     int64_t K, pt_stream_t stream);
+
+/* Rows [offs[g-1], offs[g]) of a[M,K] use b[g] of b[G,N,K]; every offs[g] is a multiple of 128.
+ * Rows at or past offs[G-1] are not written.  out bf16 [M,N].
+ * deep_gemm.m_grouped_fp8(_fp4)_gemm_nt_contiguous at grouped_linear.py:88-101 (forward :146-154,
+ * dgrad :192-200). */
+int pt_gemm_m_grouped_nt(const void* a_fp8, const float* a_scale, const void* b_fp8,
+                         const float* b_scale, void* out, int out_dtype, const int32_t* offs,
+                         int32_t num_groups, int64_t M, int64_t N, int64_t K, pt_stream_t stream);
+
+/* dW[g][n,k] = sum_{m in group g} dY[m,n] X[m,k] with colwise-quantised operands stored
+ * transposed: dy_t[N,M] and x_t[K,M] (PT_CH_TRANSPOSED) and their scales dy_scale[M/128,N],
+ * x_scale[M/128,K].  out is [G,N,K]:
+ *   out_dtype PT_F32 : fp32, accumulate==0 overwrites, !=0 adds (the `c=` operand)
+ *   out_dtype PT_BF16: bf16(sum) rounded once; accumulate!=0 then adds the existing bf16 value
+ *                      in fp32 and rounds again (weight.grad += wgrad.to(bf16)).
+ * Groups with no rows get zeros (or are left unchanged when accumulating).
+ * deep_gemm.k_grouped_fp8_gemm_{tn,nt}_contiguous + grad_weight_fn, grouped_linear.py:202-221. */
+int pt_gemm_k_grouped_wgrad(const void* dy_t_fp8, const float* dy_scale, const void* x_t_fp8,
+                            const float* x_scale, void* out, int out_dtype, int accumulate,
+                            const int32_t* offs, int32_t num_groups, int64_t M, int64_t N,
+                            int64_t K, pt_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Routing-driven permute / unpermute.  Replace pithtrain/operators/token_scatter.py.
+ * ------------------------------------------------------------------------------------------ */
+
+/* Bytes of workspace pt_group_rows needs for m keys and num_groups groups. */
+int64_t pt_group_rows_workspace_bytes(int64_t m, int32_t num_groups);
+
+/* Stable counting sort of rows by group with every group padded to `alignment` rows.
+ *   keys[m] int64 in [0,num_groups)            (expert_idxs)
+ *   offs[G] int32 inclusive cumsum of padded sizes, ks[G] int32 padded sizes
+ *   reverse[m] int64: destination row of source row i  (reverse_shuffle_idxs)
+ *   src_of[cap] int32: source row of destination row r, -1 for pad rows (r < cap)
+ * Canonical order: ascending source row inside a group.
+ * _compute_group_offsets_kernel + slot assignment of _scatter_for_grouped_gemm_kernel,
+ * token_scatter.py:38-101. */
+int pt_group_rows(const int64_t* keys, int64_t m, int32_t num_groups, int32_t alignment,
+                  int32_t* offs, int32_t* ks, int64_t* reverse, int32_t* src_of, int64_t cap,
+                  void* workspace, int64_t workspace_bytes, pt_stream_t stream);
+
+/* out[r,:] = src_of[r] >= 0 ? in[pre ? pre[src_of[r]] : src_of[r], :] : 0   for r < rows_out,
+ * where rows_out = min(cap, round_up(offs_last[0], tail_alignment)) read on the device when
+ * offs_last != NULL, else cap.  Rows in [rows_out, cap) are not touched.  elem_bytes-wide
+ * elements, H per row.  `pre` (int64, may be NULL) composes a first gather (the dedup expand)
+ * into the same pass.
+ * Row copy + pad/tail zeroing of _scatter_for_grouped_gemm_kernel, token_scatter.py:103-153. */
+int pt_permute_rows(const void* in, int64_t ld_in, void* out, int64_t ld_out, const int32_t* src_of,
+                    const int64_t* pre, const int32_t* offs_last, int32_t tail_alignment,
+                    int64_t cap, int64_t H, int32_t elem_bytes, pt_stream_t stream);
+
+/* out[i,:] = in[index[i],:], i < n.  index int64.
+ * _PaddedIndexGather.forward (token_scatter.py:297-309), ScatterForGroupedGemm.backward
+ * (:271-284). */
+int pt_gather_rows(const void* in, int64_t ld_in, void* out, int64_t ld_out, const int64_t* index,
+                   int64_t n, int64_t H, int32_t elem_bytes, pt_stream_t stream);
+
+/* Bytes of workspace pt_gather_rows_backward needs. */
+int64_t pt_gather_rows_backward_workspace_bytes(int64_t n, int64_t rows);
+
+/* grad_in[r,:] = sum over {j : index[j] == r} of grad_out[j,:], r < rows; summed in fp32 in
+ * ascending j, rounded once to the element type (dtype PT_BF16 / PT_F32 / PT_F16).
+ * _PaddedIndexGather.backward (scatter_add_), token_scatter.py:311-325. */
+int pt_gather_rows_backward(const void* grad_out, int64_t ld_go, void* grad_in, int64_t ld_gi,
+                            const int64_t* index, int64_t n, int64_t rows, int64_t H, int dtype,
+                            void* workspace, int64_t workspace_bytes, pt_stream_t stream);
+
+/* group_ids[r] = min(#{g : offs[g] <= r}, G-1), r < M; out_dtype_bytes 4 (int32) or 8 (int64).
+ * precompute_group_indices, token_scatter.py:370-384; GptOssExperts.forward,
+ * models/gpt_oss.py:146-150. */
+int pt_group_indices(const int32_t* offs, int32_t num_groups, int64_t M, void* group_ids,
+                     int32_t out_dtype_bytes, pt_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Expert-parallel dispatch index construction with token dedup.
+ * Replace the Triton kernels of pithtrain/operators/ep_dispatch.py.
+ * ------------------------------------------------------------------------------------------ */
+
+int64_t pt_dedup_workspace_bytes(int64_t m, int32_t k, int32_t num_experts, int32_t ep_size);
+
+/* topk_ids[m,k] int64 (row stride ld_ids) -> tokens_per_ep_rank[ep], dedup_tokens_per_gpu[ep],
+ * dispatch_token_idxs[m*ep] (first sum(dedup) valid), idxs[m*k], expand_idx[m*k],
+ * send_meta[ep*(epr+1)], all int64.  Canonical order: ascending flat index inside an expert
+ * bucket, ascending token id inside an EP-rank chunk.
+ * fused_dedup_prepare_dispatch, ep_dispatch.py:271-420. */
+int pt_dedup_prepare_dispatch(const int64_t* topk_ids, int64_t ld_ids, int64_t m, int32_t k,
+                              int32_t num_experts, int32_t ep_size, int32_t experts_per_rank,
+                              int64_t* tokens_per_ep_rank, int64_t* dedup_tokens_per_gpu,
+                              int64_t* dispatch_token_idxs, int64_t* idxs, int64_t* expand_idx,
+                              int64_t* send_meta, void* workspace, int64_t workspace_bytes,
+                              pt_stream_t stream);
+
+/* expert_idxs[s] = e % experts_per_rank for slot s in bucket e (s < sum(counts), s < max_total);
+ * output_splits[g] = sum of counts of rank g.   build_expert_idxs, ep_dispatch.py:426-508. */
+int pt_build_expert_idxs(const int64_t* tokens_per_expert_group, int32_t num_experts,
+                         int32_t ep_size, int32_t experts_per_rank, int64_t max_total,
+                         int64_t* expert_idxs, int64_t* output_splits, pt_stream_t stream);
+
+/* out[i] = received[i] + exclusive_cumsum(dedup_counts)[sender(i)], sender from output_splits.
+ * dedup_counts has element stride dedup_stride.   adjust_expand_idx, ep_dispatch.py:511-576. */
+int pt_adjust_expand_idx(const int64_t* received, int64_t* out, const int64_t* dedup_counts,
+                         int64_t dedup_stride, const int64_t* output_splits, int32_t ep_size,
+                         int64_t n, pt_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Fused epilogues.  dtype is the storage type (PT_BF16 / PT_F16 / PT_F32); math in fp32.
+ * ------------------------------------------------------------------------------------------ */
+
+/* out = silu(gate) * up over n elements.   _silu_mul_fwd_kernel, silu_mul.py:28-49 */
+int pt_silu_mul_fwd(const void* gate, const void* up, void* out, int64_t n, int dtype,
+                    pt_stream_t stream);
+/* _silu_mul_bwd_kernel, silu_mul.py:52-87 */
+int pt_silu_mul_bwd(const void* grad_out, const void* gate, const void* up, void* grad_gate,
+                    void* grad_up, int64_t n, int dtype, pt_stream_t stream);
+/* gate_up[M,2N] interleaved -> out[M,N]; n = M*N.  _clamped_swiglu_fwd_kernel,
+ * clamped_swiglu.py:18-46 */
+int pt_clamped_swiglu_fwd(const void* gate_up, void* out, int64_t n, float alpha, float limit,
+                          int dtype, pt_stream_t stream);
+/* _clamped_swiglu_bwd_kernel, clamped_swiglu.py:49-89 */
+int pt_clamped_swiglu_bwd(const void* grad_out, const void* gate_up, void* grad_gate_up, int64_t n,
+                          float alpha, float limit, int dtype, pt_stream_t stream);
+/* out[r,:] = x[r,:] + bias[group_ids[r],:]  (group_ids int64).  _IndexedBiasAdd.forward,
+ * indexed_bias_add.py:100-104 */
+int pt_indexed_bias_add_fwd(const void* x, const void* bias, const int64_t* group_ids, void* out,
+                            int64_t M, int64_t H, int dtype, pt_stream_t stream);
+/* out[g,:] = sum of rows [offs[g-1], min(offs[g],M)) of x, fp32 accumulate, stored as out_dtype.
+ * _segment_sum_kernel, indexed_bias_add.py:20-96 */
+int pt_segment_sum(const void* x, const int32_t* offs, int32_t num_groups, void* out, int64_t M,
+                   int64_t H, int dtype, int out_dtype, pt_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PITHTRAIN_HIP_H */

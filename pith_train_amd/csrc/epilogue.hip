@@ -1,0 +1,284 @@
+// Fused activation / bias epilogues of the expert path (HBM-bound elementwise kernels).
+//
+// Every thread moves 8 elements per step with 16-byte loads/stores (two for fp32); math is
+// fp32 with one rounding to the storage type.  Grids are sized to the element count so that a
+// launch has many more workgroups than the 256 CUs.
+#include "common.h"
+
+namespace pt {
+
+__device__ __forceinline__ float sigmoidf_fast(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+}
+
+// ---- silu_mul ---------------------------------------------------------------------------------
+template <typename S>
+__global__ __launch_bounds__(256) void silu_mul_fwd_kernel(const char* gate, const char* up, char* out, int64_t n) {
+  const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i0 >= n) return;
+  if (i0 + 8 <= n) {
+    float g[8], u[8], o[8];
+    S::load8(gate + i0 * S::kBytes, g);
+    S::load8(up + i0 * S::kBytes, u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = g[j] * sigmoidf_fast(g[j]) * u[j];
+    S::store8(out + i0 * S::kBytes, o);
+  } else {
+    for (int64_t i = i0; i < n; ++i) {
+      const float g = S::load1(gate + i * S::kBytes), u = S::load1(up + i * S::kBytes);
+      S::store1(out + i * S::kBytes, g * sigmoidf_fast(g) * u);
+    }
+  }
+}
+
+template <typename S>
+__global__ __launch_bounds__(256) void silu_mul_bwd_kernel(const char* go, const char* gate, const char* up,
+                                                           char* dgate, char* dup, int64_t n) {
+  const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i0 >= n) return;
+  auto one = [](float d, float g, float u, float& dg, float& du) {
+    const float sig = sigmoidf_fast(g);
+    const float silu = g * sig;
+    du = d * silu;
+    dg = d * u * sig * (1.0f + g - silu);
+  };
+  if (i0 + 8 <= n) {
+    float d[8], g[8], u[8], dg[8], du[8];
+    S::load8(go + i0 * S::kBytes, d);
+    S::load8(gate + i0 * S::kBytes, g);
+    S::load8(up + i0 * S::kBytes, u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) one(d[j], g[j], u[j], dg[j], du[j]);
+    S::store8(dgate + i0 * S::kBytes, dg);
+    S::store8(dup + i0 * S::kBytes, du);
+  } else {
+    for (int64_t i = i0; i < n; ++i) {
+      float dg, du;
+      one(S::load1(go + i * S::kBytes), S::load1(gate + i * S::kBytes), S::load1(up + i * S::kBytes), dg, du);
+      S::store1(dgate + i * S::kBytes, dg);
+      S::store1(dup + i * S::kBytes, du);
+    }
+  }
+}
+
+// ---- clamped SwiGLU (interleaved gate/up) ---------------------------------------------------------
+__device__ __forceinline__ float cswiglu_f(float g, float u, float alpha, float limit) {
+  const float gc = fminf(g, limit);
+  const float uc = fminf(fmaxf(u, -limit), limit);
+  return (uc + 1.0f) * (gc * sigmoidf_fast(alpha * gc));
+}
+__device__ __forceinline__ void cswiglu_b(float d, float g, float u, float alpha, float limit, float& dg, float& du) {
+  const float gc = fminf(g, limit);
+  const float uc = fminf(fmaxf(u, -limit), limit);
+  const float sig = sigmoidf_fast(alpha * gc);
+  const float glu = gc * sig;
+  const float grad_uc = d * glu;
+  const float grad_gc = d * (uc + 1.0f) * sig * (1.0f + alpha * gc * (1.0f - sig));
+  dg = (g <= limit) ? grad_gc : 0.0f;
+  du = (u >= -limit && u <= limit) ? grad_uc : 0.0f;
+}
+
+template <typename S>
+__global__ __launch_bounds__(256) void clamped_swiglu_fwd_kernel(const char* gu, char* out, int64_t n, float alpha, float limit) {
+  const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i0 >= n) return;
+  if (i0 + 8 <= n) {
+    float a[8], b[8], o[8];
+    S::load8(gu + (2 * i0) * S::kBytes, a);
+    S::load8(gu + (2 * i0 + 8) * S::kBytes, b);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      o[j] = cswiglu_f(a[2 * j], a[2 * j + 1], alpha, limit);
+      o[4 + j] = cswiglu_f(b[2 * j], b[2 * j + 1], alpha, limit);
+    }
+    S::store8(out + i0 * S::kBytes, o);
+  } else {
+    for (int64_t i = i0; i < n; ++i)
+      S::store1(out + i * S::kBytes,
+                cswiglu_f(S::load1(gu + (2 * i) * S::kBytes), S::load1(gu + (2 * i + 1) * S::kBytes), alpha, limit));
+  }
+}
+
+template <typename S>
+__global__ __launch_bounds__(256) void clamped_swiglu_bwd_kernel(const char* go, const char* gu, char* dgu, int64_t n,
+                                                                 float alpha, float limit) {
+  const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i0 >= n) return;
+  if (i0 + 8 <= n) {
+    float d[8], a[8], b[8], da[8], db[8];
+    S::load8(go + i0 * S::kBytes, d);
+    S::load8(gu + (2 * i0) * S::kBytes, a);
+    S::load8(gu + (2 * i0 + 8) * S::kBytes, b);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      cswiglu_b(d[j], a[2 * j], a[2 * j + 1], alpha, limit, da[2 * j], da[2 * j + 1]);
+      cswiglu_b(d[4 + j], b[2 * j], b[2 * j + 1], alpha, limit, db[2 * j], db[2 * j + 1]);
+    }
+    S::store8(dgu + (2 * i0) * S::kBytes, da);
+    S::store8(dgu + (2 * i0 + 8) * S::kBytes, db);
+  } else {
+    for (int64_t i = i0; i < n; ++i) {
+      float dg, du;
+      cswiglu_b(S::load1(go + i * S::kBytes), S::load1(gu + (2 * i) * S::kBytes), S::load1(gu + (2 * i + 1) * S::kBytes),
+                alpha, limit, dg, du);
+      S::store1(dgu + (2 * i) * S::kBytes, dg);
+      S::store1(dgu + (2 * i + 1) * S::kBytes, du);
+    }
+  }
+}
+
+// ---- x + bias[group_ids] -----------------------------------------------------------------------------
+template <typename S>
+__global__ __launch_bounds__(256) void bias_add_kernel(const char* x, const char* bias, const int64_t* gid, char* out,
+                                                       int64_t M, int64_t H, int vec) {
+  if (vec) {
+    const int64_t chunks = H / 8;
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= M * chunks) return;
+    const int64_t r = c / chunks, h = (c - r * chunks) * 8;
+    float a[8], b[8];
+    S::load8(x + (r * H + h) * S::kBytes, a);
+    S::load8(bias + (gid[r] * H + h) * S::kBytes, b);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) a[j] += b[j];
+    S::store8(out + (r * H + h) * S::kBytes, a);
+  } else {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= M * H) return;
+    const int64_t r = i / H, h = i - r * H;
+    S::store1(out + i * S::kBytes, S::load1(x + i * S::kBytes) + S::load1(bias + (gid[r] * H + h) * S::kBytes));
+  }
+}
+
+// ---- per-group row sums -----------------------------------------------------------------------------
+// grid (ceil(H/128), G); 16 column chunks x 16 row lanes; fp32 accumulate, fixed order.
+template <typename S, typename O>
+__global__ __launch_bounds__(256) void segment_sum_kernel(const char* x, const int32_t* offs, char* out, int64_t M,
+                                                          int64_t H, int vec) {
+  __shared__ float s[16][129];
+  const int g = blockIdx.y;
+  const int cc = threadIdx.x & 15, rl = threadIdx.x >> 4;
+  int64_t start = g == 0 ? 0 : (int64_t)offs[g - 1];
+  int64_t end = offs[g];
+  if (end > M) end = M;
+  if (start > M) start = M;
+  const int64_t h0 = (int64_t)blockIdx.x * 128 + cc * 8;
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (vec) {
+    if (h0 < H)
+      for (int64_t r = start + rl; r < end; r += 16) {
+        float v[8];
+        S::load8(x + (r * H + h0) * S::kBytes, v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] += v[j];
+      }
+  } else {
+    for (int64_t r = start + rl; r < end; r += 16)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (h0 + j < H) acc[j] += S::load1(x + (r * H + h0 + j) * S::kBytes);
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s[rl][cc * 8 + j] = acc[j];
+  __syncthreads();
+  if (threadIdx.x < 128) {
+    const int64_t h = (int64_t)blockIdx.x * 128 + threadIdx.x;
+    if (h < H) {
+      float t = 0.f;
+#pragma unroll
+      for (int q = 0; q < 16; ++q) t += s[q][threadIdx.x];
+      O::store1(out + ((int64_t)g * H + h) * O::kBytes, t);
+    }
+  }
+}
+
+static inline unsigned blocks8(int64_t n) { return (unsigned)cdiv(cdiv(n, 8), 256); }
+
+#define PT_DISPATCH_ST(dtype, NAME, ...)                                   \
+  switch (dtype) {                                                         \
+    case PT_BF16: NAME<st_bf16> __VA_ARGS__; break;                        \
+    case PT_F16:  NAME<st_f16> __VA_ARGS__; break;                         \
+    case PT_F32:  NAME<st_f32> __VA_ARGS__; break;                         \
+    default: PT_REQUIRE(false, "unsupported dtype %d", dtype);             \
+  }
+
+}  // namespace pt
+
+using namespace pt;
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+extern "C" int pt_silu_mul_fwd(const void* gate, const void* up, void* out, int64_t n, int dtype, pt_stream_t stream) {
+  if (n == 0) return PT_OK;
+  PT_REQUIRE(n > 0 && gate && up && out, "silu_mul_fwd: bad arguments");
+  PT_REQUIRE(aligned16(gate) && aligned16(up) && aligned16(out), "silu_mul_fwd: pointers must be 16-byte aligned");
+  PT_REQUIRE(cdiv(n, 2048) < (1ll << 31), "silu_mul_fwd: too many elements");
+  hipStream_t s = (hipStream_t)stream;
+  PT_DISPATCH_ST(dtype, silu_mul_fwd_kernel, <<<blocks8(n), 256, 0, s>>>((const char*)gate, (const char*)up, (char*)out, n));
+  return check_launch("silu_mul_fwd");
+}
+
+extern "C" int pt_silu_mul_bwd(const void* go, const void* gate, const void* up, void* dgate, void* dup, int64_t n,
+                               int dtype, pt_stream_t stream) {
+  if (n == 0) return PT_OK;
+  PT_REQUIRE(n > 0 && go && gate && up && dgate && dup, "silu_mul_bwd: bad arguments");
+  PT_REQUIRE(aligned16(go) && aligned16(gate) && aligned16(up) && aligned16(dgate) && aligned16(dup),
+             "silu_mul_bwd: pointers must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  PT_DISPATCH_ST(dtype, silu_mul_bwd_kernel,
+                 <<<blocks8(n), 256, 0, s>>>((const char*)go, (const char*)gate, (const char*)up, (char*)dgate, (char*)dup, n));
+  return check_launch("silu_mul_bwd");
+}
+
+extern "C" int pt_clamped_swiglu_fwd(const void* gate_up, void* out, int64_t n, float alpha, float limit, int dtype,
+                                     pt_stream_t stream) {
+  if (n == 0) return PT_OK;
+  PT_REQUIRE(n > 0 && gate_up && out, "clamped_swiglu_fwd: bad arguments");
+  PT_REQUIRE(aligned16(gate_up) && aligned16(out), "clamped_swiglu_fwd: pointers must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  PT_DISPATCH_ST(dtype, clamped_swiglu_fwd_kernel, <<<blocks8(n), 256, 0, s>>>((const char*)gate_up, (char*)out, n, alpha, limit));
+  return check_launch("clamped_swiglu_fwd");
+}
+
+extern "C" int pt_clamped_swiglu_bwd(const void* go, const void* gate_up, void* dgu, int64_t n, float alpha, float limit,
+                                     int dtype, pt_stream_t stream) {
+  if (n == 0) return PT_OK;
+  PT_REQUIRE(n > 0 && go && gate_up && dgu, "clamped_swiglu_bwd: bad arguments");
+  PT_REQUIRE(aligned16(go) && aligned16(gate_up) && aligned16(dgu), "clamped_swiglu_bwd: pointers must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  PT_DISPATCH_ST(dtype, clamped_swiglu_bwd_kernel,
+                 <<<blocks8(n), 256, 0, s>>>((const char*)go, (const char*)gate_up, (char*)dgu, n, alpha, limit));
+  return check_launch("clamped_swiglu_bwd");
+}
+
+extern "C" int pt_indexed_bias_add_fwd(const void* x, const void* bias, const int64_t* group_ids, void* out, int64_t M,
+                                       int64_t H, int dtype, pt_stream_t stream) {
+  if (M == 0 || H == 0) return PT_OK;
+  PT_REQUIRE(M > 0 && H > 0 && x && bias && group_ids && out, "indexed_bias_add_fwd: bad arguments");
+  const int vec = (H % 8 == 0) && aligned16(x) && aligned16(bias) && aligned16(out);
+  const int64_t work = vec ? M * (H / 8) : M * H;
+  PT_REQUIRE(cdiv(work, 256) < (1ll << 31), "indexed_bias_add_fwd: too many elements");
+  hipStream_t s = (hipStream_t)stream;
+  PT_DISPATCH_ST(dtype, bias_add_kernel,
+                 <<<(unsigned)cdiv(work, 256), 256, 0, s>>>((const char*)x, (const char*)bias, group_ids, (char*)out, M, H, vec));
+  return check_launch("indexed_bias_add_fwd");
+}
+
+extern "C" int pt_segment_sum(const void* x, const int32_t* offs, int32_t num_groups, void* out, int64_t M, int64_t H,
+                              int dtype, int out_dtype, pt_stream_t stream) {
+  if (num_groups == 0 || H == 0) return PT_OK;
+  PT_REQUIRE(num_groups > 0 && num_groups <= 65535 && H > 0 && M >= 0 && x && offs && out, "segment_sum: bad arguments");
+  const int vec = (H % 8 == 0) && aligned16(x);
+  dim3 grid((unsigned)cdiv(H, 128), (unsigned)num_groups);
+  hipStream_t s = (hipStream_t)stream;
+#define PT_SEG(SI, SO) segment_sum_kernel<SI, SO><<<grid, 256, 0, s>>>((const char*)x, offs, (char*)out, M, H, vec)
+  if (dtype == PT_BF16 && out_dtype == PT_BF16) PT_SEG(st_bf16, st_bf16);
+  else if (dtype == PT_BF16 && out_dtype == PT_F32) PT_SEG(st_bf16, st_f32);
+  else if (dtype == PT_F16 && out_dtype == PT_F16) PT_SEG(st_f16, st_f16);
+  else if (dtype == PT_F16 && out_dtype == PT_F32) PT_SEG(st_f16, st_f32);
+  else if (dtype == PT_F32 && out_dtype == PT_F32) PT_SEG(st_f32, st_f32);
+  else if (dtype == PT_F32 && out_dtype == PT_BF16) PT_SEG(st_f32, st_bf16);
+  else PT_REQUIRE(false, "segment_sum: unsupported dtype pair %d -> %d", dtype, out_dtype);
+#undef PT_SEG
+  return check_launch("segment_sum");
+}

@@ -1,0 +1,346 @@
+// FP8 (e4m3) GEMMs on the gfx950 matrix cores with hardware block scaling.
+//
+// One kernel template serves the three GEMM shapes of the expert path:
+//   dense      out[m,n]      = sum_k a[m,k] b[n,k]
+//   m-grouped  out[rows_g,n] = a[rows_g,:] . b[g][n,:]            (forward, dgrad)
+//   k-grouped  out[g][n,k]   = sum_{m in g} dy_t[n,m] x_t[k,m]     (wgrad)
+// All are "NT": both operands are contiguous along the reduction dimension.  Every scale of
+// this path is an exact power of two, so it is handed to v_mfma_scale_f32_32x32x64_f8f6f4 as
+// an E8M0 exponent byte and applied inside the MFMA: one fp32 accumulator runs over the whole
+// reduction and no VALU promotion step is needed.
+//
+// Workgroup = BM x BN output tile, 128-deep reduction steps (one scale block).  Operand tiles go
+// global -> LDS with 16-byte direct-to-LDS loads (no VGPR staging), double buffered; 16-byte
+// chunks are XOR-swizzled by choosing which global chunk each lane fetches, so the later
+// ds_read_b128 fragment reads are spread over the banks.  Per step a wave reads all of its
+// fragments, then the next tile's loads are issued, then the MFMAs run while those loads land.
+#include "common.h"
+
+namespace pt {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+enum { GEMM_DENSE = 0, GEMM_M_GROUPED = 1, GEMM_K_GROUPED = 2 };
+
+struct GemmArgs {
+  const uint8_t* a; int64_t lda;          // [rows_a, red] bytes
+  const uint8_t* b; int64_t ldb;          // [rows_b, red] bytes
+  const float* sa; int64_t sa_rs, sa_ks; int sa_shift;  // scale(row,kb) = sa[(row>>shift)*rs + kb*ks]
+  const float* sb; int64_t sb_rs, sb_ks; int sb_shift;
+  void* out; int64_t ldo;                 // elements
+  int out_dtype; int accumulate;
+  int64_t rows_a, rows_b, red;            // output is rows_a x rows_b; red = reduction length (dense / m-grouped)
+  const int32_t* offs; int G;
+  int mode;
+  int64_t b_stride_g, sb_stride_g, out_stride_g;
+  int tiles_a, tiles_b;                   // tile counts along rows_a / rows_b
+  int64_t total_tiles;
+};
+
+__device__ __attribute__((aligned(16))) uint32_t g_zero_chunk[4] = {0, 0, 0, 0};
+
+__device__ __forceinline__ void load_lds16(const uint8_t* g, uint8_t* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                   (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
+template <int BM, int BN, int WGM, int WGN>
+__global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_nt_kernel(GemmArgs p) {
+  constexpr int NW = WGM * WGN;
+  constexpr int WM = BM / WGM, WN = BN / WGN;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;  // direct-to-LDS wave loads per step
+  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/wave mismatch");
+  constexpr int STAGE = (BM + BN) * 128;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  __shared__ int s_cnt[NW];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
+
+  // ---- which tile: consecutive logical tiles stay on one XCD (workgroups are dealt round-robin
+  // over the 8 XCDs), and inside a group the tiles that share a b-tile are adjacent ----
+  const int64_t per_xcd = (p.total_tiles + 7) / 8;
+  const int64_t t = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (t >= p.total_tiles) return;
+
+  int64_t a_row0, b_row0, a_lim, b_lim, k_begin, k_end, kb0;
+  const uint8_t* bp = p.b;
+  const float* sbp = p.sb;
+  char* outp = (char*)p.out;
+  if (p.mode == GEMM_DENSE) {
+    const int ta = (int)(t % p.tiles_a), tb = (int)(t / p.tiles_a);
+    a_row0 = (int64_t)ta * BM; b_row0 = (int64_t)tb * BN;
+    a_lim = p.rows_a; b_lim = p.rows_b; k_begin = 0; k_end = p.red; kb0 = 0;
+  } else if (p.mode == GEMM_M_GROUPED) {
+    // row tile index in group-major order; groups are multiples of 128 rows and BM == 128
+    const int64_t tr = t / p.tiles_b;
+    const int64_t row = tr * BM;
+    int cnt = 0;
+    for (int g = tid; g < p.G; g += NW * 64) cnt += ((int64_t)p.offs[g] <= row) ? 1 : 0;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) cnt += __shfl_xor(cnt, d);
+    if (lane == 0) s_cnt[wave] = cnt;
+    __syncthreads();
+    int g = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) g += s_cnt[w];
+    if (g >= p.G) return;  // rows past the last group
+    const int64_t gs = g == 0 ? 0 : p.offs[g - 1], ge = p.offs[g];
+    const int64_t m_tiles = (ge - gs) / BM, first = (gs / BM) * p.tiles_b;
+    const int64_t idx = t - first;
+    const int tb = (int)(idx / m_tiles);
+    a_row0 = gs + (idx % m_tiles) * BM; b_row0 = (int64_t)tb * BN;
+    a_lim = ge; b_lim = p.rows_b; k_begin = 0; k_end = p.red; kb0 = 0;
+    bp += (int64_t)g * p.b_stride_g; sbp += (int64_t)g * p.sb_stride_g;
+  } else {
+    const int64_t per_g = (int64_t)p.tiles_a * p.tiles_b;
+    const int g = (int)(t / per_g);
+    const int64_t idx = t % per_g;
+    const int ta = (int)(idx % p.tiles_a), tb = (int)(idx / p.tiles_a);
+    a_row0 = (int64_t)ta * BM; b_row0 = (int64_t)tb * BN;
+    a_lim = p.rows_a; b_lim = p.rows_b;
+    k_begin = g == 0 ? 0 : p.offs[g - 1]; k_end = p.offs[g]; kb0 = k_begin >> 7;
+    outp += (int64_t)g * p.out_stride_g * (p.out_dtype == PT_F32 ? 4 : 2);
+  }
+  const int nk = (int)((k_end - k_begin + 127) >> 7);
+
+  // ---- per-lane global source pointers of the direct-to-LDS loads ----
+  // wave-load q covers tile rows 8*(wave + NW*q) .. +8; lane -> row +lane/8, physical chunk lane%8,
+  // which holds logical chunk (lane%8) ^ f(row), f(row) = (row&7) ^ ((row>>3)&1).
+  const int lrow = lane >> 3;
+  const int lchunk = (lane & 7) ^ lrow ^ (wave & 1);
+  const uint8_t* ap[LA];
+  const uint8_t* bpp[LB];
+#pragma unroll
+  for (int q = 0; q < LA; ++q) {
+    int64_t r = a_row0 + 8 * (wave + NW * q) + lrow;
+    if (r >= a_lim) r = a_lim - 1;
+    ap[q] = p.a + r * p.lda + k_begin + lchunk * 16;
+  }
+#pragma unroll
+  for (int q = 0; q < LB; ++q) {
+    int64_t r = b_row0 + 8 * (wave + NW * q) + lrow;
+    if (r >= b_lim) r = b_lim - 1;
+    bpp[q] = bp + r * p.ldb + k_begin + lchunk * 16;
+  }
+  const int64_t k_len = k_end - k_begin;
+  const uint8_t* zero = (const uint8_t*)g_zero_chunk;
+
+  auto issue_loads = [&](int it, int stage) {
+    uint8_t* sA = lds + stage * STAGE;
+    uint8_t* sB = sA + BM * 128;
+    const int64_t koff = (int64_t)it * 128;
+    const bool in = koff + lchunk * 16 < k_len;  // false only in a ragged last step
+#pragma unroll
+    for (int q = 0; q < LA; ++q) load_lds16(in ? ap[q] + koff : zero, sA + (wave + NW * q) * 1024);
+#pragma unroll
+    for (int q = 0; q < LB; ++q) load_lds16(in ? bpp[q] + koff : zero, sB + (wave + NW * q) * 1024);
+  };
+
+  // ---- per-lane scale sources ----
+  int64_t sa_idx[TM], sb_idx[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    int64_t r = a_row0 + wm0 + i * 32 + (lane & 31);
+    if (r >= a_lim) r = a_lim - 1;
+    sa_idx[i] = (r >> p.sa_shift) * p.sa_rs + kb0 * p.sa_ks;
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int64_t r = b_row0 + wn0 + j * 32 + (lane & 31);
+    if (r >= b_lim) r = b_lim - 1;
+    sb_idx[j] = (r >> p.sb_shift) * p.sb_rs + kb0 * p.sb_ks;
+  }
+
+  v16f acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // fragment read offsets inside a tile (lane-constant): row (lane&31), chunk (ks*4 + (lane>>5)*2 + h) ^ f
+  const int f = (lane & 7) ^ ((lane >> 3) & 1);
+  const int roff = (lane & 31) * 128;
+  int coff[2][2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) coff[ks][h] = roff + (((ks * 4 + (lane >> 5) * 2 + h) ^ f) << 4);
+
+  // Scales of step `it` are fetched (raw fp32 bits) one step ahead, before that step's tile loads
+  // are issued, and only turned into E8M0 bytes after the next barrier: nothing between a step's
+  // loads and its MFMAs waits on the vector-memory counter.
+  float raw_a[TM], raw_b[TN];
+  if (nk > 0) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) raw_a[i] = p.sa[sa_idx[i]];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) raw_b[j] = sbp[sb_idx[j]];
+    issue_loads(0, 0);
+  }
+
+  for (int it = 0; it < nk; ++it) {
+    const int stage = it & 1;
+    // Every wave drains its own direct-to-LDS loads *before* the barrier: the workgroup fence of
+    // __syncthreads() does not wait on the vector-memory counter, and the other waves are about
+    // to read the rows this wave fetched.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    int sca[TM], scb[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) sca[i] = (int)(__float_as_uint(raw_a[i]) >> 23);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) scb[j] = (int)(__float_as_uint(raw_b[j]) >> 23);
+    const uint8_t* sA = lds + stage * STAGE + wm0 * 128;
+    const uint8_t* sB = lds + stage * STAGE + BM * 128 + wn0 * 128;
+    v8i af[2][TM], bf[2][TN];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const uint4 lo = *(const uint4*)(sA + i * 4096 + coff[ks][0]);
+        const uint4 hi = *(const uint4*)(sA + i * 4096 + coff[ks][1]);
+        af[ks][i] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const uint4 lo = *(const uint4*)(sB + j * 4096 + coff[ks][0]);
+        const uint4 hi = *(const uint4*)(sB + j * 4096 + coff[ks][1]);
+        bf[ks][j] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+      }
+    }
+    if (it + 1 < nk) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) raw_a[i] = p.sa[sa_idx[i] + (int64_t)(it + 1) * p.sa_ks];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) raw_b[j] = sbp[sb_idx[j] + (int64_t)(it + 1) * p.sb_ks];
+      issue_loads(it + 1, stage ^ 1);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[ks][i], bf[ks][j], acc[i][j], 0, 0, 0, sca[i], 0,
+                                                                     scb[j]);
+  }
+
+  // ---- epilogue: lane holds column (lane&31), rows 8*(v/4) + 4*(lane>>5) + (v&3) of each 32x32 ----
+  if (p.mode == GEMM_K_GROUPED && nk == 0 && p.accumulate) return;
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int64_t col = b_row0 + wn0 + j * 32 + (lane & 31);
+      if (col >= b_lim) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t row = a_row0 + wm0 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (row >= a_lim) continue;
+        const float x = acc[i][j][v];
+        if (p.out_dtype == PT_F32) {
+          float* o = (float*)outp + row * p.ldo + col;
+          *o = p.accumulate ? (*o + x) : x;
+        } else {
+          uint16_t* o = (uint16_t*)outp + row * p.ldo + col;
+          uint32_t r = f32_to_bf16_bits(x);
+          if (p.accumulate) r = f32_to_bf16_bits(bf16_bits_to_f32(*o) + bf16_bits_to_f32(r));
+          *o = (uint16_t)r;
+        }
+      }
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN>
+static int launch_gemm(const GemmArgs& a, hipStream_t stream) {
+  if (a.total_tiles == 0) return PT_OK;
+  constexpr int threads = WGM * WGN * 64;
+  constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)fp8_gemm_nt_kernel<BM, BN, WGM, WGN>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_error("gemm: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); return PT_ERR_LAUNCH; }
+    attr_set = true;
+  }
+  const int64_t per_xcd = (a.total_tiles + 7) / 8;
+  const int64_t blocks = per_xcd * 8;
+  PT_REQUIRE(blocks < (1ll << 31), "gemm: grid too large");
+  hipLaunchKernelGGL((fp8_gemm_nt_kernel<BM, BN, WGM, WGN>), dim3((unsigned)blocks), dim3(threads), lds, stream, a);
+  return check_launch("fp8_gemm_nt_kernel");
+}
+
+}  // namespace pt
+
+using namespace pt;
+
+static bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+extern "C" int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale, void* out,
+                                int out_dtype, int64_t M, int64_t N, int64_t K, pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_nt_dense: negative size");
+  if (M == 0 || N == 0) return PT_OK;
+  PT_REQUIRE(K > 0 && K % 16 == 0, "gemm_nt_dense: K=%lld must be a positive multiple of 16", (long long)K);
+  PT_REQUIRE(a_fp8 && a_scale && b_fp8 && b_scale && out && al16(a_fp8) && al16(b_fp8), "gemm_nt_dense: null or misaligned pointer");
+  PT_REQUIRE(out_dtype == PT_BF16 || out_dtype == PT_F32, "gemm_nt_dense: out_dtype must be bf16 or fp32");
+  const int64_t KB = cdiv(K, 128);
+  GemmArgs g = {};
+  g.a = (const uint8_t*)a_fp8; g.lda = K; g.b = (const uint8_t*)b_fp8; g.ldb = K;
+  g.sa = a_scale; g.sa_rs = KB; g.sa_ks = 1; g.sa_shift = 0;
+  g.sb = b_scale; g.sb_rs = KB; g.sb_ks = 1; g.sb_shift = 7;
+  g.out = out; g.ldo = N; g.out_dtype = out_dtype; g.accumulate = 0;
+  g.rows_a = M; g.rows_b = N; g.red = K; g.mode = GEMM_DENSE;
+  g.tiles_a = (int)cdiv(M, 128); g.tiles_b = (int)cdiv(N, 128);
+  g.total_tiles = (int64_t)g.tiles_a * g.tiles_b;
+  return launch_gemm<128, 128, 2, 2>(g, (hipStream_t)stream);
+}
+
+extern "C" int pt_gemm_m_grouped_nt(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
+                                    void* out, int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N, int64_t K,
+                                    pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && N >= 0 && K >= 0 && G > 0, "gemm_m_grouped_nt: bad sizes");
+  if (M == 0 || N == 0) return PT_OK;
+  PT_REQUIRE(M % 128 == 0, "gemm_m_grouped_nt: M=%lld must be a multiple of 128", (long long)M);
+  PT_REQUIRE(K > 0 && K % 16 == 0, "gemm_m_grouped_nt: K=%lld must be a positive multiple of 16", (long long)K);
+  PT_REQUIRE(a_fp8 && a_scale && b_fp8 && b_scale && out && offs && al16(a_fp8) && al16(b_fp8), "gemm_m_grouped_nt: null or misaligned pointer");
+  PT_REQUIRE(out_dtype == PT_BF16, "gemm_m_grouped_nt: out_dtype must be bf16");
+  PT_REQUIRE((N * K) % 16 == 0, "gemm_m_grouped_nt: N*K must be a multiple of 16");
+  const int64_t KB = cdiv(K, 128), NB = cdiv(N, 128);
+  GemmArgs g = {};
+  g.a = (const uint8_t*)a_fp8; g.lda = K; g.b = (const uint8_t*)b_fp8; g.ldb = K;
+  g.sa = a_scale; g.sa_rs = KB; g.sa_ks = 1; g.sa_shift = 0;
+  g.sb = b_scale; g.sb_rs = KB; g.sb_ks = 1; g.sb_shift = 7;
+  g.out = out; g.ldo = N; g.out_dtype = out_dtype; g.accumulate = 0;
+  g.rows_a = M; g.rows_b = N; g.red = K; g.mode = GEMM_M_GROUPED; g.offs = offs; g.G = G;
+  g.b_stride_g = N * K; g.sb_stride_g = NB * KB;
+  g.tiles_a = (int)(M / 128); g.tiles_b = (int)NB;
+  g.total_tiles = (int64_t)g.tiles_a * g.tiles_b;
+  return launch_gemm<128, 128, 2, 2>(g, (hipStream_t)stream);
+}
+
+extern "C" int pt_gemm_k_grouped_wgrad(const void* dy_t_fp8, const float* dy_scale, const void* x_t_fp8, const float* x_scale,
+                                       void* out, int out_dtype, int accumulate, const int32_t* offs, int32_t G, int64_t M,
+                                       int64_t N, int64_t K, pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && N >= 0 && K >= 0 && G > 0, "gemm_k_grouped_wgrad: bad sizes");
+  if (N == 0 || K == 0) return PT_OK;
+  PT_REQUIRE(M % 128 == 0, "gemm_k_grouped_wgrad: M=%lld must be a multiple of 128", (long long)M);
+  PT_REQUIRE(out && offs, "gemm_k_grouped_wgrad: null pointer");
+  PT_REQUIRE(M == 0 || (dy_t_fp8 && dy_scale && x_t_fp8 && x_scale && al16(dy_t_fp8) && al16(x_t_fp8)),
+             "gemm_k_grouped_wgrad: null or misaligned pointer");
+  PT_REQUIRE(out_dtype == PT_BF16 || out_dtype == PT_F32, "gemm_k_grouped_wgrad: out_dtype must be bf16 or fp32");
+  GemmArgs g = {};
+  g.a = (const uint8_t*)dy_t_fp8; g.lda = M; g.b = (const uint8_t*)x_t_fp8; g.ldb = M;
+  g.sa = dy_scale; g.sa_rs = 1; g.sa_ks = N; g.sa_shift = 0;
+  g.sb = x_scale; g.sb_rs = 1; g.sb_ks = K; g.sb_shift = 0;
+  g.out = out; g.ldo = K; g.out_dtype = out_dtype; g.accumulate = accumulate;
+  g.rows_a = N; g.rows_b = K; g.red = M; g.mode = GEMM_K_GROUPED; g.offs = offs; g.G = G;
+  g.out_stride_g = N * K;
+  g.tiles_a = (int)cdiv(N, 128); g.tiles_b = (int)cdiv(K, 128);
+  g.total_tiles = (int64_t)g.tiles_a * g.tiles_b * G;
+  return launch_gemm<128, 128, 2, 2>(g, (hipStream_t)stream);
+}

@@ -1,0 +1,364 @@
+// Blockwise FP8 quantisation kernels for gfx950.
+//
+// One workgroup (256 threads, 4 wavefronts) owns one 128x128 tile of the source: it is read
+// once with 16-byte loads, reduced three ways (per row, per column, whole tile) and written as
+// up to two e4m3 tensors plus their power-of-two scales.  Thread t holds the 8x8 sub-block at
+// rows (t/16)*8.., columns (t%16)*8.. so that a 16-lane DPP row covers one 128-column row
+// segment (row amax is a DPP all-reduce) and one thread owns 8 consecutive rows of each of its
+// columns (so transposed bytes can be packed straight from registers).  Transposed twins go
+// through an XOR-swizzled LDS tile so that global stores are 16 bytes wide and 128-byte
+// contiguous per 8 lanes.  The kernel is HBM-bound: 2 (or 4) bytes in, 2 bytes out per element.
+#include "common.h"
+
+namespace pt {
+
+enum { A_ROW = 0, A_BLOCK = 1 };                       // scaling of the same-orientation output
+enum { B_COL = 0, B_BLOCK = 1 };                       // scaling of the twin
+enum { BL_ROWMAJOR = 0, BL_TRANSPOSED = 1, BL_KMAJOR = 2 };  // layout of the twin's bytes
+enum { BS_MB_N = 0, BS_N_MB = 1 };                     // twin scale layout for B_COL
+
+struct QuantArgs {
+  const void* x;
+  int64_t M, N, ldx, x_stride_g;
+  uint8_t* a_out;  int64_t a_stride_g;   // [M,N] bytes, ld = N
+  float* a_scale;  int64_t a_scale_stride_g;
+  uint8_t* b_out;  int64_t b_stride_g;   // rowmajor [M,N] / transposed [N,M] / kmajor flat
+  float* b_scale;  int64_t b_scale_stride_g;
+  int32_t tiles_m, tiles_n;
+  const int32_t* offs; int32_t num_groups;  // KMAJOR only
+  int32_t vec_in;     // 16-byte loads legal (alignment + N % 8 == 0)
+  int32_t vec_out;    // 8-byte row-major stores legal (N % 8 == 0)
+  int32_t vec_out_t;  // 16-byte transposed stores legal
+};
+
+template <typename T> struct Loader;
+struct bf16_tag {};
+template <> struct Loader<bf16_tag> {
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ void load8(const void* p, float* v) {
+    const uint4 u = *reinterpret_cast<const uint4*>(p);
+    v[0] = bf16_lo(u.x); v[1] = bf16_hi(u.x); v[2] = bf16_lo(u.y); v[3] = bf16_hi(u.y);
+    v[4] = bf16_lo(u.z); v[5] = bf16_hi(u.z); v[6] = bf16_lo(u.w); v[7] = bf16_hi(u.w);
+  }
+  static __device__ __forceinline__ float load1(const void* p) {
+    return bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(p));
+  }
+};
+template <> struct Loader<float> {
+  static constexpr int kBytes = 4;
+  static __device__ __forceinline__ void load8(const void* p, float* v) {
+    const float4 a = reinterpret_cast<const float4*>(p)[0];
+    const float4 b = reinterpret_cast<const float4*>(p)[1];
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  static __device__ __forceinline__ float load1(const void* p) {
+    return *reinterpret_cast<const float*>(p);
+  }
+};
+
+template <typename T, int AM, int BMODE, int BL, int BS>
+__global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
+  __shared__ float s_colmax[4][128];
+  __shared__ float s_blk[4];
+  __shared__ __attribute__((aligned(16))) uint8_t s_t[128 * 128];
+
+  const int t = threadIdx.x;
+  const int cc = t & 15, rg = t >> 4, wave = t >> 6, lane = t & 63;
+  int64_t bid = blockIdx.x;
+  const int tc = (int)(bid % p.tiles_n); bid /= p.tiles_n;
+  const int tr = (int)(bid % p.tiles_m);
+  const int64_t g = bid / p.tiles_m;
+
+  const int64_t row0 = (int64_t)tr * 128 + rg * 8;
+  const int64_t col0 = (int64_t)tc * 128 + cc * 8;
+  const char* xb = reinterpret_cast<const char*>(p.x) + g * p.x_stride_g * Loader<T>::kBytes;
+
+  float v[8][8];
+  if (p.vec_in) {
+    const bool col_ok = col0 < p.N;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (col_ok && row0 + i < p.M) {
+        Loader<T>::load8(xb + ((row0 + i) * p.ldx + col0) * Loader<T>::kBytes, v[i]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[i][j] = 0.f;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        v[i][j] = (row0 + i < p.M && col0 + j < p.N)
+                      ? Loader<T>::load1(xb + ((row0 + i) * p.ldx + col0 + j) * Loader<T>::kBytes)
+                      : 0.f;
+  }
+
+  // ---- reductions ------------------------------------------------------------------------
+  float rowmax[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float m = fabsf(v[i][0]);
+#pragma unroll
+    for (int j = 1; j < 8; ++j) m = fmaxf(m, fabsf(v[i][j]));
+    rowmax[i] = m;
+  }
+  if (AM == A_ROW) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) rowmax[i] = row16_allmax(rowmax[i]);
+  }
+
+  float colmax[8];
+  if (BMODE == B_COL) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float m = fabsf(v[0][j]);
+#pragma unroll
+      for (int i = 1; i < 8; ++i) m = fmaxf(m, fabsf(v[i][j]));
+      m = fmaxf(m, __shfl_xor(m, 16));
+      m = fmaxf(m, __shfl_xor(m, 32));
+      colmax[j] = m;
+    }
+    if (lane < 16) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s_colmax[wave][cc * 8 + j] = colmax[j];
+    }
+  }
+  float blkmax = 0.f;
+  if (AM == A_BLOCK || BMODE == B_BLOCK) {
+    float m = rowmax[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) m = fmaxf(m, rowmax[i]);
+    if (AM != A_ROW) m = row16_allmax(m);
+    m = fmaxf(m, __shfl_xor(m, 16));
+    m = fmaxf(m, __shfl_xor(m, 32));
+    if (lane == 0) s_blk[wave] = m;
+  }
+  __syncthreads();
+  if (BMODE == B_COL) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      colmax[j] = fmaxf(fmaxf(s_colmax[0][cc * 8 + j], s_colmax[1][cc * 8 + j]),
+                        fmaxf(s_colmax[2][cc * 8 + j], s_colmax[3][cc * 8 + j]));
+  }
+  float blk_scale = 0.f, blk_rcp = 0.f;
+  if (AM == A_BLOCK || BMODE == B_BLOCK) {
+    blkmax = fmaxf(fmaxf(s_blk[0], s_blk[1]), fmaxf(s_blk[2], s_blk[3]));
+    blk_scale = fp8_scale_from_amax(blkmax, blk_rcp);
+  }
+
+  // ---- same-orientation output -----------------------------------------------------------
+  {
+    uint8_t* ab = p.a_out + g * p.a_stride_g;
+    const int64_t nb = p.tiles_n;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float rcp;
+      if (AM == A_ROW) {
+        const float s = fp8_scale_from_amax(rowmax[i], rcp);
+        if (cc == 0 && row0 + i < p.M) p.a_scale[(row0 + i) * nb + tc] = s;
+      } else {
+        rcp = blk_rcp;
+      }
+      const uint32_t lo = cvt4_e4m3(v[i][0] * rcp, v[i][1] * rcp, v[i][2] * rcp, v[i][3] * rcp);
+      const uint32_t hi = cvt4_e4m3(v[i][4] * rcp, v[i][5] * rcp, v[i][6] * rcp, v[i][7] * rcp);
+      if (row0 + i < p.M) {
+        uint8_t* dst = ab + (row0 + i) * p.N + col0;
+        if (p.vec_out) {
+          if (col0 < p.N) *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (col0 + j < p.N) dst[j] = (uint8_t)(((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xFF);
+        }
+      }
+    }
+    if (AM == A_BLOCK && t == 0)
+      p.a_scale[g * p.a_scale_stride_g + (int64_t)tr * p.tiles_n + tc] = blk_scale;
+  }
+
+  // ---- twin ---------------------------------------------------------------------------------
+  float crcp[8];
+  if (BMODE == B_COL) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float s = fp8_scale_from_amax(colmax[j], crcp[j]);
+      if (rg == 0 && col0 + j < p.N) {
+        if (BS == BS_MB_N) p.b_scale[(int64_t)tr * p.N + col0 + j] = s;
+        else               p.b_scale[(col0 + j) * (int64_t)p.tiles_m + tr] = s;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) crcp[j] = blk_rcp;
+    if (t == 0) p.b_scale[g * p.b_scale_stride_g + (int64_t)tc * p.tiles_m + tr] = blk_scale;
+  }
+
+  if (BL == BL_ROWMAJOR) {
+    uint8_t* bb = p.b_out + g * p.b_stride_g;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t lo = cvt4_e4m3(v[i][0] * crcp[0], v[i][1] * crcp[1], v[i][2] * crcp[2], v[i][3] * crcp[3]);
+      const uint32_t hi = cvt4_e4m3(v[i][4] * crcp[4], v[i][5] * crcp[5], v[i][6] * crcp[6], v[i][7] * crcp[7]);
+      if (row0 + i < p.M) {
+        uint8_t* dst = bb + (row0 + i) * p.N + col0;
+        if (p.vec_out) {
+          if (col0 < p.N) *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (col0 + j < p.N) dst[j] = (uint8_t)(((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xFF);
+        }
+      }
+    }
+  } else {
+    // pack 8 consecutive rows of each column and stage the transposed tile in LDS:
+    // s_t[n][m], 16-byte chunk index XOR-swizzled with (n >> 3) & 7.
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float r = crcp[j];
+      const uint32_t lo = cvt4_e4m3(v[0][j] * r, v[1][j] * r, v[2][j] * r, v[3][j] * r);
+      const uint32_t hi = cvt4_e4m3(v[4][j] * r, v[5][j] * r, v[6][j] * r, v[7][j] * r);
+      const int n = cc * 8 + j;
+      const int chunk = (rg >> 1) ^ ((n >> 3) & 7);
+      *reinterpret_cast<uint2*>(&s_t[n * 128 + chunk * 16 + (rg & 1) * 8]) = make_uint2(lo, hi);
+    }
+    __syncthreads();
+    // destination of tile element (n, m): base + n * ld + m
+    uint8_t* base;
+    int64_t ld;
+    if (BL == BL_TRANSPOSED) {
+      base = p.b_out + g * p.b_stride_g + (int64_t)tc * 128 * p.M + (int64_t)tr * 128;
+      ld = p.M;
+    } else {
+      const int64_t row_start = (int64_t)tr * 128;
+      int grp = 0;
+      int64_t gstart = 0, gend = 0;
+      for (int q = 0; q < p.num_groups; ++q) {  // uniform scalar scan; groups are 128-aligned
+        const int64_t e = p.offs[q];
+        if (e <= row_start && q < p.num_groups - 1) { grp = q + 1; gstart = e; }
+      }
+      gend = p.offs[grp];
+      (void)gend;
+      const int64_t kg = (int64_t)p.offs[grp] - gstart;
+      base = p.b_out + gstart * p.N + (int64_t)tc * 128 * kg + (row_start - gstart);
+      ld = kg;
+    }
+    const int mc = t & 7;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int n = (t >> 3) + 32 * k;
+      const int64_t gn = (int64_t)tc * 128 + n;
+      const int64_t gm = (int64_t)tr * 128 + mc * 16;
+      if (gn >= p.N) continue;
+      const uint4 val = *reinterpret_cast<const uint4*>(&s_t[n * 128 + ((mc ^ ((n >> 3) & 7)) * 16)]);
+      uint8_t* dst = base + n * ld + mc * 16;
+      if (p.vec_out_t) {
+        if (gm < p.M) *reinterpret_cast<uint4*>(dst) = val;
+      } else {
+        const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+        for (int b = 0; b < 16; ++b)
+          if (gm + b < p.M) dst[b] = (uint8_t)((w[b >> 2] >> (8 * (b & 3))) & 0xFF);
+      }
+    }
+  }
+}
+
+template <int AM, int BMODE, int BL, int BS>
+static int launch_quant(const QuantArgs& a, int dtype, int64_t G, hipStream_t stream) {
+  const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n * G;
+  if (blocks == 0) return PT_OK;
+  PT_REQUIRE(blocks < (1ll << 31), "quant: grid too large (%lld tiles)", (long long)blocks);
+  if (dtype == PT_BF16)
+    hipLaunchKernelGGL((quant_tile_kernel<bf16_tag, AM, BMODE, BL, BS>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else if (dtype == PT_F32)
+    hipLaunchKernelGGL((quant_tile_kernel<float, AM, BMODE, BL, BS>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else
+    PT_REQUIRE(false, "quant: unsupported dtype %d (bf16 and fp32 only)", dtype);
+  return check_launch("quant_tile_kernel");
+}
+
+static void fill_common(QuantArgs& a, const void* x, int dtype, int64_t M, int64_t N, int64_t ldx) {
+  a.x = x; a.M = M; a.N = N; a.ldx = ldx; a.x_stride_g = 0;
+  a.a_stride_g = 0; a.a_scale_stride_g = 0; a.b_stride_g = 0; a.b_scale_stride_g = 0;
+  a.tiles_m = (int32_t)cdiv(M, 128); a.tiles_n = (int32_t)cdiv(N, 128);
+  a.offs = nullptr; a.num_groups = 0;
+  const int eb = dtype == PT_F32 ? 4 : 2;
+  a.vec_in = (N % 8 == 0) && ((ldx * eb) % 16 == 0) && (((uintptr_t)x) % 16 == 0);
+  a.vec_out = (N % 8 == 0);
+  a.vec_out_t = (M % 16 == 0);
+}
+
+}  // namespace pt
+
+using namespace pt;
+
+extern "C" int pt_quant_rowwise_colwise(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
+                                        void* tok_fp8, float* tok_scale, void* ch_fp8,
+                                        float* ch_scale, int ch_layout, const int32_t* offs,
+                                        int32_t num_groups, pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && N >= 0 && M % 128 == 0, "quant_rowwise_colwise: M=%lld must be a multiple of 128", (long long)M);
+  PT_REQUIRE(ldx >= N, "quant_rowwise_colwise: ldx < N");
+  if (M == 0 || N == 0) return PT_OK;
+  PT_REQUIRE(x && tok_fp8 && tok_scale && ch_fp8 && ch_scale, "quant_rowwise_colwise: null pointer");
+  QuantArgs a;
+  fill_common(a, x, dtype, M, N, ldx);
+  a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)ch_fp8; a.b_scale = ch_scale;
+  hipStream_t s = (hipStream_t)stream;
+  switch (ch_layout) {
+    case PT_CH_ROWMAJOR:   return launch_quant<A_ROW, B_COL, BL_ROWMAJOR, BS_MB_N>(a, dtype, 1, s);
+    case PT_CH_TRANSPOSED: return launch_quant<A_ROW, B_COL, BL_TRANSPOSED, BS_MB_N>(a, dtype, 1, s);
+    case PT_CH_KMAJOR:
+      PT_REQUIRE(offs && num_groups > 0, "quant_rowwise_colwise: kmajor layout needs offs");
+      a.offs = offs; a.num_groups = num_groups;
+      return launch_quant<A_ROW, B_COL, BL_KMAJOR, BS_N_MB>(a, dtype, 1, s);
+  }
+  PT_REQUIRE(false, "quant_rowwise_colwise: bad ch_layout %d", ch_layout);
+}
+
+extern "C" int pt_quant_rowwise_transpose(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
+                                          void* tok_fp8, float* tok_scale, void* t_fp8,
+                                          float* t_scale, pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && N >= 0 && ldx >= N, "quant_rowwise_transpose: bad shape");
+  if (M == 0 || N == 0) return PT_OK;
+  PT_REQUIRE(x && tok_fp8 && tok_scale && t_fp8 && t_scale, "quant_rowwise_transpose: null pointer");
+  QuantArgs a;
+  fill_common(a, x, dtype, M, N, ldx);
+  a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)t_fp8; a.b_scale = t_scale;
+  return launch_quant<A_ROW, B_COL, BL_TRANSPOSED, BS_N_MB>(a, dtype, 1, (hipStream_t)stream);
+}
+
+extern "C" int pt_quant_rowwise_blockwise_transpose(const void* x, int dtype, int64_t M, int64_t K,
+                                                    int64_t ldx, void* tok_fp8, float* tok_scale,
+                                                    void* blk_t_fp8, float* blk_t_scale,
+                                                    pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && K >= 0 && ldx >= K, "quant_rowwise_blockwise_transpose: bad shape");
+  if (M == 0 || K == 0) return PT_OK;
+  PT_REQUIRE(x && tok_fp8 && tok_scale && blk_t_fp8 && blk_t_scale, "quant_rowwise_blockwise_transpose: null pointer");
+  QuantArgs a;
+  fill_common(a, x, dtype, M, K, ldx);
+  a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)blk_t_fp8; a.b_scale = blk_t_scale;
+  return launch_quant<A_ROW, B_BLOCK, BL_TRANSPOSED, BS_MB_N>(a, dtype, 1, (hipStream_t)stream);
+}
+
+extern "C" int pt_quant_blockwise_transpose_batched(const void* x, int dtype, int64_t G, int64_t N,
+                                                    int64_t K, int64_t stride_g, int64_t stride_row,
+                                                    void* fp8, float* scale, void* fp8_t,
+                                                    float* scale_t, pt_stream_t stream) {
+  PT_REQUIRE(G >= 0 && N >= 0 && K >= 0 && stride_row >= K, "quant_blockwise_transpose_batched: bad shape");
+  if (G == 0 || N == 0 || K == 0) return PT_OK;
+  PT_REQUIRE(x && fp8 && scale && fp8_t && scale_t, "quant_blockwise_transpose_batched: null pointer");
+  QuantArgs a;
+  fill_common(a, x, dtype, N, K, stride_row);
+  const int eb = dtype == PT_F32 ? 4 : 2;
+  a.vec_in = a.vec_in && ((stride_g * eb) % 16 == 0);
+  a.x_stride_g = stride_g;
+  a.a_out = (uint8_t*)fp8; a.a_stride_g = N * K; a.a_scale = scale; a.a_scale_stride_g = (int64_t)a.tiles_m * a.tiles_n;
+  a.b_out = (uint8_t*)fp8_t; a.b_stride_g = N * K; a.b_scale = scale_t; a.b_scale_stride_g = (int64_t)a.tiles_m * a.tiles_n;
+  // transposed stores of group g start at g*N*K: 16-byte alignment needs (N*K) % 16 == 0 too
+  a.vec_out_t = a.vec_out_t && ((N * K) % 16 == 0);
+  a.vec_out = a.vec_out && ((N * K) % 8 == 0);
+  return launch_quant<A_BLOCK, B_BLOCK, BL_TRANSPOSED, BS_MB_N>(a, dtype, G, (hipStream_t)stream);
+}

@@ -1,0 +1,149 @@
+"""Expert blocks of the supported model families and the stage-3 composition around them.
+
+Mirrors the expert path of the reference's model files:
+  * ``Qwen3MoeExperts``      - models/qwen3_moe.py:45-65   (gate, up, down as three grouped linears)
+  * ``DeepSeekV2Experts``    - models/deepseek_v2.py:111-129
+  * ``DeepSeekV2MLP``        - models/deepseek_v2.py:94-108 (dense shared expert)
+  * ``Qwen35MoeExperts``     - models/qwen35_moe.py:179-200 (fused gate_up, concatenated halves)
+  * ``GptOssExperts``        - models/gpt_oss.py:95-157     (fused interleaved gate_up, biases,
+                                                              clamped SwiGLU)
+  * ``forward_stage3``       - models/qwen3_moe.py:216-227  (expand -> scatter -> experts -> gather)
+
+The constructors take plain sizes instead of Hugging Face config objects; everything else
+(parameter names, shapes, call signatures) follows the reference so that checkpoints and callers
+line up.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from ..dualpipe_utils import FP8WeightCacheControl
+from ..operators.clamped_swiglu import clamped_swiglu
+from ..operators.deepgemm_quantize import fp8cast_blockwise_transpose_batched
+from ..operators.grouped_linear import FP8GroupedLinearFunc, GroupedLinearFunc
+from ..operators.indexed_bias_add import indexed_bias_add
+from ..operators.silu_mul import silu_mul
+from ..operators.token_scatter import (
+    group_indices,
+    padded_index_gather,
+    precompute_group_indices,
+    scatter_for_grouped_gemm,
+)
+from . import training
+
+
+class Qwen3MoeExperts(nn.Module):
+    def __init__(self, hidden_size: int, moe_intermediate_size: int, num_experts: int):
+        super().__init__()
+        self.gate_proj = training.GroupedLinear(num_experts, hidden_size, moe_intermediate_size)
+        self.up_proj = training.GroupedLinear(num_experts, hidden_size, moe_intermediate_size)
+        self.down_proj = training.GroupedLinear(num_experts, moe_intermediate_size, hidden_size)
+
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None):
+        gi = precompute_group_indices(grouped_mm_offs, x.shape[0])
+        kwargs = dict(grouped_mm_offs=grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, group_indices=gi)
+        g = self.gate_proj(x, **kwargs)
+        u = self.up_proj(x, **kwargs)
+        return self.down_proj(silu_mul(g, u), **kwargs)
+
+
+class DeepSeekV2Experts(Qwen3MoeExperts):
+    """Same composition as the Qwen3 experts (models/deepseek_v2.py:111-129)."""
+
+
+class DeepSeekV2MLP(nn.Module):
+    """Dense SwiGLU MLP (the shared experts run as one of these)."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        super().__init__()
+        self.gate_proj = training.Linear(hidden_size, intermediate_size, bias=False)
+        self.up_proj = training.Linear(hidden_size, intermediate_size, bias=False)
+        self.down_proj = training.Linear(intermediate_size, hidden_size, bias=False)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.down_proj(silu_mul(self.gate_proj(x), self.up_proj(x)))
+
+
+class Qwen35MoeExperts(nn.Module):
+    def __init__(self, hidden_size: int, moe_intermediate_size: int, num_experts: int):
+        super().__init__()
+        self.num_experts = num_experts
+        self.hidden_size = hidden_size
+        self.moe_intermediate_size = moe_intermediate_size
+        self.gate_up_proj = training.GroupedLinear(num_experts, hidden_size, 2 * moe_intermediate_size)
+        self.down_proj = training.GroupedLinear(num_experts, moe_intermediate_size, hidden_size)
+
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None):
+        gi = precompute_group_indices(grouped_mm_offs, x.shape[0])
+        kwargs = dict(grouped_mm_offs=grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, group_indices=gi)
+        gate_up = self.gate_up_proj(x, **kwargs)
+        gate = gate_up[:, : self.moe_intermediate_size].contiguous()
+        up = gate_up[:, self.moe_intermediate_size :].contiguous()
+        return self.down_proj(silu_mul(gate, up), **kwargs)
+
+
+class GptOssExperts(nn.Module):
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, swiglu_limit: float = 7.0):
+        super().__init__()
+        self.num_experts = num_experts
+        self.swiglu_limit = float(swiglu_limit)
+        self.gate_up_proj = nn.Parameter(torch.empty(num_experts, 2 * intermediate_size, hidden_size))
+        self.gate_up_proj_bias = nn.Parameter(torch.zeros(num_experts, 2 * intermediate_size))
+        self.down_proj = nn.Parameter(torch.empty(num_experts, hidden_size, intermediate_size))
+        self.down_proj_bias = nn.Parameter(torch.zeros(num_experts, hidden_size))
+        self._wq_cache: dict | None = None
+        self._wq_version: int = -1
+
+    def _quantized_weight(self, name: str, weight: torch.Tensor):
+        if torch.compiler.is_compiling():
+            return fp8cast_blockwise_transpose_batched(weight)
+        ver = FP8WeightCacheControl.version
+        cache = self._wq_cache
+        if self._wq_version != ver or cache is None:
+            cache = self._wq_cache = {}
+            self._wq_version = ver
+        if name not in cache:
+            cache[name] = fp8cast_blockwise_transpose_batched(weight)
+        return cache[name]
+
+    def _group_linear(self, x, weight, name, offs, ks, ks_tensor, group_indices_):
+        if x.shape[0] == 0:
+            return x @ weight[0].transpose(-2, -1)
+        if training.fp8:
+            return FP8GroupedLinearFunc.apply(
+                x, weight, offs, ks, ks_tensor, self._quantized_weight(name, weight), group_indices_
+            )
+        return GroupedLinearFunc.apply(x, weight, offs)
+
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None):
+        group_ids = group_indices(grouped_mm_offs, x.shape[0], torch.int64)
+        gate_up = self._group_linear(x, self.gate_up_proj, "gate_up_proj", grouped_mm_offs, ks, ks_tensor, None)
+        gate_up = indexed_bias_add(gate_up, self.gate_up_proj_bias, group_ids, grouped_mm_offs)
+        activated = clamped_swiglu(gate_up, 1.702, self.swiglu_limit)
+        out = self._group_linear(activated, self.down_proj, "down_proj", grouped_mm_offs, ks, ks_tensor, None)
+        return indexed_bias_add(out, self.down_proj_bias, group_ids, grouped_mm_offs)
+
+
+def forward_stage3(experts: nn.Module, gathered_tokens, expert_idxs, experts_per_rank: int, expand_idx=None,
+                   fuse_expand: bool = True):
+    """Expert compute between the dispatch and combine all-to-alls.
+
+    ``expand_idx`` (EP > 1) re-expands the deduplicated received rows to one row per routed
+    (token, expert) pair.  With ``fuse_expand`` that gather is folded into the scatter's row copy
+    (each unique row is read once per use and no expanded copy is materialised); without it the
+    two steps run separately as in the reference.
+    """
+    pre = None
+    if expand_idx is not None:
+        if fuse_expand:
+            pre = expand_idx
+        else:
+            gathered_tokens = padded_index_gather(gathered_tokens, expand_idx)
+    output_tokens, reverse_shuffle_idxs, grouped_mm_offs, ks, ks_tensor = scatter_for_grouped_gemm(
+        gathered_tokens, expert_idxs, experts_per_rank, pre_index=pre
+    )
+    del gathered_tokens
+    outs = experts(output_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor)
+    return padded_index_gather(outs, reverse_shuffle_idxs)

@@ -1,0 +1,153 @@
+"""Blockwise FP8 quantisation (e4m3fn, power-of-two fp32 scales) on gfx950.
+
+Drop-in for ``pithtrain/operators/deepgemm_quantize.py``: same six entry points, same return
+tuples, layouts and dtypes (``:16-23``).  ``fp8cast_rowwise_colwise_t`` is this package's own
+variant that stores the colwise twin transposed, which is the operand layout of the wgrad GEMM
+here.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+__all__ = [
+    "fp8cast_rowwise_colwise",
+    "fp8cast_rowwise_kmajor",
+    "fp8cast_rowwise_transpose",
+    "fp8cast_rowwise_blockwise_transpose",
+    "fp8cast_blockwise_transpose",
+    "fp8cast_blockwise_transpose_batched",
+    "fp8cast_rowwise_colwise_t",
+]
+
+FP8 = torch.float8_e4m3fn
+
+
+def _prep2d(x: torch.Tensor) -> torch.Tensor:
+    _lib.require_cuda(x)
+    if x.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"fp8cast: expected bfloat16 or float32 input, got {x.dtype}")
+    if x.shape[-1] > 0 and x.stride(-1) != 1:
+        x = x.contiguous()
+    return x
+
+
+def _cdiv(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def _rowwise_colwise(x: torch.Tensor, layout: int, offs: torch.Tensor | None):
+    assert x.ndim == 2 and x.shape[0] % 128 == 0, (
+        f"Expected 2D tensor with M%128==0, got shape {tuple(x.shape)}"
+    )
+    x = _prep2d(x)
+    M, N = x.shape
+    dev = x.device
+    out_tok = torch.empty((M, N), dtype=FP8, device=dev)
+    scale_tok = torch.empty((M, _cdiv(N, 128)), dtype=torch.float32, device=dev)
+    if layout == _lib.PT_CH_ROWMAJOR:
+        out_ch = torch.empty((M, N), dtype=FP8, device=dev)
+        scale_ch = torch.empty((M // 128, N), dtype=torch.float32, device=dev)
+    elif layout == _lib.PT_CH_TRANSPOSED:
+        out_ch = torch.empty((N, M), dtype=FP8, device=dev)
+        scale_ch = torch.empty((M // 128, N), dtype=torch.float32, device=dev)
+    else:
+        out_ch = torch.empty(M * N, dtype=FP8, device=dev)
+        scale_ch = torch.empty((N, M // 128), dtype=torch.float32, device=dev)
+    if M == 0 or N == 0:
+        return out_tok, scale_tok, out_ch, scale_ch
+    ld = x.stride(0) if M > 1 else N
+    _lib.call(
+        "pt_quant_rowwise_colwise", x.data_ptr(), _lib.dtype_code(x.dtype), M, N, ld,
+        out_tok.data_ptr(), scale_tok.data_ptr(), out_ch.data_ptr(), scale_ch.data_ptr(), layout,
+        _lib.ptr(offs), 0 if offs is None else offs.shape[0], _lib.stream_ptr(dev),
+    )  # fmt: skip
+    return out_tok, scale_tok, out_ch, scale_ch
+
+
+def fp8cast_rowwise_colwise(x: torch.Tensor):
+    """(tok_fp8[M,N], tok_scale[M,ceil(N/128)], ch_fp8[M,N], ch_scale[M//128,N]); M % 128 == 0."""
+    return _rowwise_colwise(x, _lib.PT_CH_ROWMAJOR, None)
+
+
+def fp8cast_rowwise_colwise_t(x: torch.Tensor):
+    """As :func:`fp8cast_rowwise_colwise` with the colwise bytes stored transposed: ch_t_fp8[N,M]
+    (``ch_t_fp8 == ch_fp8.T`` byte for byte), ch_scale[M//128,N] unchanged."""
+    return _rowwise_colwise(x, _lib.PT_CH_TRANSPOSED, None)
+
+
+def fp8cast_rowwise_kmajor(x: torch.Tensor, grouped_mm_offs: torch.Tensor):
+    """Rowwise outputs as above; colwise bytes per group as (N, K_g) blocks in a flat 1-D buffer,
+    colwise scales transposed to (N, M//128)."""
+    assert grouped_mm_offs.dtype == torch.int32 and grouped_mm_offs.ndim == 1
+    return _rowwise_colwise(x, _lib.PT_CH_KMAJOR, grouped_mm_offs.contiguous())
+
+
+def fp8cast_rowwise_transpose(x: torch.Tensor):
+    """(tok_fp8[M,N], tok_scale[M,ceil(N/128)], t_fp8[N,M], t_scale[N,ceil(M/128)])."""
+    assert x.ndim == 2, f"Expected 2D tensor, got {x.ndim}D"
+    x = _prep2d(x)
+    M, N = x.shape
+    dev = x.device
+    out_tok = torch.empty((M, N), dtype=FP8, device=dev)
+    scale_tok = torch.empty((M, _cdiv(N, 128)), dtype=torch.float32, device=dev)
+    out_t = torch.empty((N, M), dtype=FP8, device=dev)
+    scale_t = torch.empty((N, _cdiv(M, 128)), dtype=torch.float32, device=dev)
+    if M and N:
+        _lib.call(
+            "pt_quant_rowwise_transpose", x.data_ptr(), _lib.dtype_code(x.dtype), M, N,
+            x.stride(0) if M > 1 else N, out_tok.data_ptr(), scale_tok.data_ptr(), out_t.data_ptr(),
+            scale_t.data_ptr(), _lib.stream_ptr(dev),
+        )  # fmt: skip
+    return out_tok, scale_tok, out_t, scale_t
+
+
+def fp8cast_rowwise_blockwise_transpose(x: torch.Tensor):
+    """(tok_fp8[M,K], tok_scale[M,ceil(K/128)], blk_t_fp8[K,M], blk_t_scale[ceil(K/128),ceil(M/128)])."""
+    assert x.ndim == 2, f"Expected 2D tensor, got {x.ndim}D"
+    x = _prep2d(x)
+    M, K = x.shape
+    dev = x.device
+    out_tok = torch.empty((M, K), dtype=FP8, device=dev)
+    scale_tok = torch.empty((M, _cdiv(K, 128)), dtype=torch.float32, device=dev)
+    out_blk_t = torch.empty((K, M), dtype=FP8, device=dev)
+    scale_blk_t = torch.empty((_cdiv(K, 128), _cdiv(M, 128)), dtype=torch.float32, device=dev)
+    if M and K:
+        _lib.call(
+            "pt_quant_rowwise_blockwise_transpose", x.data_ptr(), _lib.dtype_code(x.dtype), M, K,
+            x.stride(0) if M > 1 else K, out_tok.data_ptr(), scale_tok.data_ptr(),
+            out_blk_t.data_ptr(), scale_blk_t.data_ptr(), _lib.stream_ptr(dev),
+        )  # fmt: skip
+    return out_tok, scale_tok, out_blk_t, scale_blk_t
+
+
+def _blockwise_batched(x3: torch.Tensor):
+    G, N, K = x3.shape
+    dev = x3.device
+    out = torch.empty((G, N, K), dtype=FP8, device=dev)
+    scale = torch.empty((G, _cdiv(N, 128), _cdiv(K, 128)), dtype=torch.float32, device=dev)
+    out_t = torch.empty((G, K, N), dtype=FP8, device=dev)
+    scale_t = torch.empty((G, _cdiv(K, 128), _cdiv(N, 128)), dtype=torch.float32, device=dev)
+    if G and N and K:
+        _lib.call(
+            "pt_quant_blockwise_transpose_batched", x3.data_ptr(), _lib.dtype_code(x3.dtype), G, N, K,
+            x3.stride(0) if G > 1 else N * K, x3.stride(1) if N > 1 else K, out.data_ptr(),
+            scale.data_ptr(), out_t.data_ptr(), scale_t.data_ptr(), _lib.stream_ptr(dev),
+        )  # fmt: skip
+    return out, scale, out_t, scale_t
+
+
+def fp8cast_blockwise_transpose(x: torch.Tensor):
+    """(fp8[M,K], scale[ceil(M/128),ceil(K/128)], fp8_t[K,M], scale_t[ceil(K/128),ceil(M/128)])."""
+    assert x.ndim == 2, f"Expected 2D tensor, got {x.ndim}D"
+    x = _prep2d(x.detach())
+    out, scale, out_t, scale_t = _blockwise_batched(x.unsqueeze(0))
+    return out[0], scale[0], out_t[0], scale_t[0]
+
+
+def fp8cast_blockwise_transpose_batched(x: torch.Tensor):
+    """(fp8[G,N,K], scale[G,ceil(N/128),ceil(K/128)], fp8_t[G,K,N], scale_t[G,ceil(K/128),ceil(N/128)])."""
+    assert x.ndim == 3, f"Expected 3D tensor, got {x.ndim}D"
+    return _blockwise_batched(_prep2d(x.detach()))

@@ -1,0 +1,241 @@
+"""Grouped (per-expert) linear layers: FP8 on the gfx950 matrix cores, and the BF16 baseline.
+
+Drop-in for ``pithtrain/operators/grouped_linear.py``: ``GroupedLinearFunc`` / ``GroupedLinear``
+(:18-85) and ``FP8GroupedLinearFunc`` / ``FP8GroupedLinear`` (:104-284) keep their signatures,
+including the deferred weight-gradient closure handed to ``WeightGradStore`` and the direct write
+to ``weight.grad``.
+
+Differences that stay behind the interface:
+  * the colwise copies kept for the wgrad GEMM are stored transposed ([N, M]); that is the operand
+    layout of ``pt_gemm_k_grouped_wgrad``;
+  * the wgrad GEMM rounds to bf16 and (when ``weight.grad`` exists) accumulates in its epilogue,
+    instead of fp32 zeros -> GEMM -> cast -> add as four passes over a [G, N, K] tensor;
+  * ``group_indices`` is accepted and ignored (the kernels search ``grouped_mm_offs`` themselves).
+"""
+
+from __future__ import annotations
+
+from functools import partial
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .. import _lib
+from ..dualpipe_utils import FP8WeightCacheControl, WeightGradStore
+from .deepgemm_quantize import fp8cast_blockwise_transpose_batched, fp8cast_rowwise_colwise_t
+
+
+def _grouped_mm(a: torch.Tensor, b: torch.Tensor, offs: torch.Tensor) -> torch.Tensor:
+    """``F.grouped_mm`` where torch provides it, otherwise the per-group loop it stands for."""
+    if hasattr(F, "grouped_mm"):
+        try:
+            return F.grouped_mm(a, b, offs=offs)
+        except (RuntimeError, NotImplementedError):
+            pass
+    bounds = [0] + offs.tolist()
+    if a.dim() == 2 and b.dim() == 3:  # jagged on rows of a
+        out = a.new_zeros((a.shape[0], b.shape[2]))
+        for g in range(b.shape[0]):
+            s, e = bounds[g], bounds[g + 1]
+            if e > s:
+                out[s:e] = a[s:e] @ b[g]
+        return out
+    out = a.new_zeros((len(bounds) - 1, a.shape[0], b.shape[1]))  # jagged on the reduction dim
+    for g in range(len(bounds) - 1):
+        s, e = bounds[g], bounds[g + 1]
+        if e > s:
+            out[g] = a[:, s:e] @ b[s:e]
+    return out
+
+
+class GroupedLinearFunc(torch.autograd.Function):
+    """BF16 grouped linear; wgrad split off so it can be deferred (grouped_linear.py:18-55)."""
+
+    @staticmethod
+    def forward(ctx, input: torch.Tensor, weight: torch.Tensor, grouped_mm_offs: torch.Tensor):
+        output = _grouped_mm(input, weight.transpose(1, 2), grouped_mm_offs)
+        ctx.save_for_backward(input, weight, grouped_mm_offs)
+        return output
+
+    @staticmethod
+    def backward(ctx, dy):
+        input, weight, offs = ctx.saved_tensors
+        dgrad = _grouped_mm(dy, weight, offs)
+
+        def wgrad_fn(dy, x, offs):
+            wgrad = _grouped_mm(dy.transpose(0, 1), x, offs)
+            weight.grad = wgrad if weight.grad is None else weight.grad.add_(wgrad)
+
+        if WeightGradStore.enabled:
+            WeightGradStore.put(partial(wgrad_fn, dy.detach(), input.detach(), offs.detach()))
+        else:
+            wgrad_fn(dy, input, offs)
+        return dgrad, None, None
+
+
+class GroupedLinear(nn.Module):
+    """One linear map per group of rows (MoE experts), BF16."""
+
+    def __init__(self, num_groups: int, in_features: int, out_features: int):
+        super().__init__()
+        self.num_groups = num_groups
+        self.in_features = in_features
+        self.out_features = out_features
+        self.weight = nn.Parameter(torch.empty((num_groups, out_features, in_features)))
+
+    def forward(
+        self,
+        input: torch.Tensor,
+        grouped_mm_offs: torch.Tensor,
+        ks: Optional[list] = None,
+        ks_tensor: Optional[torch.Tensor] = None,
+        group_indices: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        if input.shape[0] == 0:
+            return input @ self.weight[0].T  # keeps a grad_fn with zero rows
+        return GroupedLinearFunc.apply(input, self.weight, grouped_mm_offs)
+
+
+# ------------------------------------------------------------------------------------------------
+# FP8
+# ------------------------------------------------------------------------------------------------
+def m_grouped_fp8_gemm_nt(a, b, out: torch.Tensor, grouped_mm_offs: torch.Tensor) -> torch.Tensor:
+    """out[rows_g] = a[rows_g] @ b[g].T with a=(fp8[M,K], scale[M,K/128]), b=(fp8[G,N,K],
+    scale[G,N/128,K/128]).  Rows at or past ``grouped_mm_offs[-1]`` are left untouched."""
+    (a_fp8, a_s), (b_fp8, b_s) = a, b
+    M, K = a_fp8.shape
+    G, N, _ = b_fp8.shape
+    _lib.call(
+        "pt_gemm_m_grouped_nt", a_fp8.data_ptr(), a_s.data_ptr(), b_fp8.data_ptr(), b_s.data_ptr(),
+        out.data_ptr(), _lib.dtype_code(out.dtype), grouped_mm_offs.data_ptr(), G, M, N, K,
+        _lib.stream_ptr(out.device),
+    )  # fmt: skip
+    return out
+
+
+def k_grouped_fp8_wgrad(dy_t, x_t, out: torch.Tensor, grouped_mm_offs, accumulate: bool):
+    """out[g] (+)= dY_g^T X_g with dy_t=(fp8[N,M], scale[M/128,N]), x_t=(fp8[K,M], scale[M/128,K])."""
+    (dy_fp8, dy_s), (x_fp8, x_s) = dy_t, x_t
+    N, M = dy_fp8.shape
+    K = x_fp8.shape[0]
+    G = out.shape[0]
+    _lib.call(
+        "pt_gemm_k_grouped_wgrad", dy_fp8.data_ptr(), dy_s.data_ptr(), x_fp8.data_ptr(),
+        x_s.data_ptr(), out.data_ptr(), _lib.dtype_code(out.dtype), int(accumulate),
+        grouped_mm_offs.data_ptr(), G, M, N, K, _lib.stream_ptr(out.device),
+    )  # fmt: skip
+    return out
+
+
+class FP8GroupedLinearFunc(torch.autograd.Function):
+    """FP8 grouped linear (grouped_linear.py:104-236): forward and dgrad are m-grouped NT GEMMs on
+    1x128-scaled activations against 128x128-scaled weights, wgrad a k-grouped GEMM on the colwise
+    copies."""
+
+    @staticmethod
+    def forward(
+        ctx,
+        input: torch.Tensor,
+        weight: torch.Tensor,
+        grouped_mm_offs: torch.Tensor,
+        ks: list,
+        ks_tensor: torch.Tensor,
+        quantized_weight: tuple,
+        group_indices: torch.Tensor | None = None,
+    ):
+        weight_fp8, scale_weight, weight_t_fp8, scale_weight_t = quantized_weight
+        M, K = input.shape
+        num_groups, N, _ = weight.shape
+        input_fp8, scale_input, input_ch_t, scale_input_ch = fp8cast_rowwise_colwise_t(input)
+        output = torch.empty((M, N), device=input.device, dtype=input.dtype)
+        m_grouped_fp8_gemm_nt(
+            (input_fp8, scale_input), (weight_fp8, scale_weight), output, grouped_mm_offs
+        )
+        ctx.save_for_backward(
+            weight_t_fp8, scale_weight_t, grouped_mm_offs, input_ch_t, scale_input_ch, ks_tensor
+        )
+        ctx.weight_ref = weight
+        ctx.ks = ks
+        ctx.dims = (M, K, N, num_groups)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        weight_t_fp8, scale_weight_t, offs, input_ch_t, scale_input_ch, ks_tensor = ctx.saved_tensors
+        weight = ctx.weight_ref
+        M, K, N, num_groups = ctx.dims
+        grad_output = grad_output.contiguous()
+        grad_fp8, scale_grad, grad_ch_t, scale_grad_ch = fp8cast_rowwise_colwise_t(grad_output)
+
+        grad_input = torch.empty((M, K), device=grad_output.device, dtype=grad_output.dtype)
+        m_grouped_fp8_gemm_nt((grad_fp8, scale_grad), (weight_t_fp8, scale_weight_t), grad_input, offs)
+
+        def grad_weight_fn(a, b, offs):
+            # bf16(sum) is formed in the GEMM epilogue; an existing grad is accumulated there too
+            if weight.grad is None:
+                wg = torch.empty((num_groups, N, K), device=a[0].device, dtype=torch.bfloat16)
+                k_grouped_fp8_wgrad(a, b, wg, offs, accumulate=False)
+                weight.grad = wg if weight.dtype == torch.bfloat16 else wg.to(weight.dtype)
+            elif weight.grad.dtype == torch.bfloat16 and weight.grad.is_contiguous():
+                k_grouped_fp8_wgrad(a, b, weight.grad, offs, accumulate=True)
+            else:
+                wg = torch.empty((num_groups, N, K), device=a[0].device, dtype=torch.bfloat16)
+                k_grouped_fp8_wgrad(a, b, wg, offs, accumulate=False)
+                weight.grad += wg
+
+        a_wgrad = (grad_ch_t, scale_grad_ch)
+        b_wgrad = (input_ch_t, scale_input_ch)
+        if WeightGradStore.enabled:
+            WeightGradStore.put(
+                partial(
+                    grad_weight_fn,
+                    (a_wgrad[0].detach(), a_wgrad[1].detach()),
+                    (b_wgrad[0].detach(), b_wgrad[1].detach()),
+                    offs.detach(),
+                )
+            )
+        else:
+            grad_weight_fn(a_wgrad, b_wgrad, offs)
+        return grad_input, None, None, None, None, None, None
+
+
+class FP8GroupedLinear(nn.Module):
+    """FP8 grouped linear for MoE experts; weight ``(num_groups, out_features, in_features)``.
+    The quantised weight is cached per ``FP8WeightCacheControl.version``."""
+
+    def __init__(self, num_groups: int, in_features: int, out_features: int):
+        super().__init__()
+        self.num_groups = num_groups
+        self.in_features = in_features
+        self.out_features = out_features
+        self.weight = nn.Parameter(torch.empty((num_groups, out_features, in_features)))
+        self._wq_cache = None
+        self._wq_version: int = -1
+
+    def _get_quantized_weight(self):
+        if torch.compiler.is_compiling():
+            return fp8cast_blockwise_transpose_batched(self.weight)
+        ver = FP8WeightCacheControl.version
+        if self._wq_version == ver and self._wq_cache is not None:
+            return self._wq_cache
+        result = fp8cast_blockwise_transpose_batched(self.weight)
+        self._wq_cache = result
+        self._wq_version = ver
+        return result
+
+    def forward(
+        self,
+        input: torch.Tensor,
+        grouped_mm_offs: torch.Tensor,
+        ks: list | None = None,
+        ks_tensor: torch.Tensor | None = None,
+        group_indices: torch.Tensor | None = None,
+    ) -> torch.Tensor:
+        if input.shape[0] == 0:
+            return input @ self.weight[0].T  # keeps a grad_fn with zero rows
+        return FP8GroupedLinearFunc.apply(
+            input, self.weight, grouped_mm_offs, ks, ks_tensor, self._get_quantized_weight(),
+            group_indices,
+        )  # fmt: skip

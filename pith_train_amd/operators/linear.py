@@ -1,0 +1,160 @@
+"""Dense FP8 linear on gfx950 and the shared forward / backward GEMM recipe.
+
+Drop-in for ``pithtrain/operators/linear.py``: ``fp8_act_weight_gemm`` (:44-60),
+``fp8_dgrad_wgrad`` (:63-83), the custom ops ``fp8_linear_fwd`` / ``fp8_linear_bwd`` with fake
+kernels so compiled regions can trace through them (:86-167) and ``FP8Linear`` (:170-208).  All
+three GEMMs are "1x128-scaled rows times 128x128-scaled rows, NT".
+"""
+
+from __future__ import annotations
+
+from typing import Tuple
+
+import torch
+import torch.nn as nn
+
+from .. import _lib
+from ..dualpipe_utils import FP8WeightCacheControl
+from .deepgemm_quantize import (
+    fp8cast_blockwise_transpose,
+    fp8cast_rowwise_blockwise_transpose,
+    fp8cast_rowwise_transpose,
+)
+
+# Kept for importers of the reference module (``from ...linear import ARCH_MAJOR``); nothing in
+# this package branches on it.
+ARCH_MAJOR = 9
+
+
+def _fp8_gemm_nt(a_fp8, a_scale, b_fp8, b_scale, m: int, n: int, device, dtype) -> torch.Tensor:
+    """out[m, n] = a @ b.T; a: 1x128 scales, b: 128x128 scales."""
+    k = a_fp8.shape[1]
+    out_dtype = dtype if dtype in (torch.bfloat16, torch.float32) else torch.float32
+    out = torch.empty((m, n), device=device, dtype=out_dtype)
+    _lib.call(
+        "pt_gemm_nt_dense", a_fp8.data_ptr(), a_scale.data_ptr(), b_fp8.data_ptr(),
+        b_scale.data_ptr(), out.data_ptr(), _lib.dtype_code(out_dtype), m, n, k,
+        _lib.stream_ptr(device),
+    )  # fmt: skip
+    return out if out_dtype == dtype else out.to(dtype)
+
+
+def fp8_act_weight_gemm(input_2d, weight_fp8, scale_weight):
+    """y = x @ W.T; returns (output, input_t_fp8[K,M], scale_input_t) - the transposed activation
+    is handed back for the later wgrad."""
+    m, n = input_2d.shape[0], weight_fp8.shape[0]
+    input_fp8, scale_input, input_t_fp8, scale_input_t = fp8cast_rowwise_blockwise_transpose(input_2d)
+    output = _fp8_gemm_nt(
+        input_fp8, scale_input, weight_fp8, scale_weight, m, n, input_2d.device, input_2d.dtype
+    )
+    return output, input_t_fp8, scale_input_t
+
+
+def fp8_dgrad_wgrad(grad_2d, weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t, k: int):
+    """grad_input = grad @ W (through W^T) and weight_grad = grad^T @ x (through x^T), both in
+    ``grad_2d``'s dtype."""
+    m, n = grad_2d.shape
+    grad_fp8, scale_grad, grad_t_fp8, scale_grad_t = fp8cast_rowwise_transpose(grad_2d)
+    grad_input = _fp8_gemm_nt(
+        grad_fp8, scale_grad, weight_t_fp8, scale_weight_t, m, k, grad_2d.device, grad_2d.dtype
+    )
+    weight_grad = _fp8_gemm_nt(
+        grad_t_fp8, scale_grad_t, input_t_fp8, scale_input_t, n, k, grad_2d.device, grad_2d.dtype
+    )
+    return grad_input, weight_grad
+
+
+@torch.library.custom_op("pith_train_amd::fp8_linear_fwd", mutates_args=())
+def _fp8_linear_fwd(
+    input_2d: torch.Tensor,
+    weight: torch.Tensor,
+    weight_fp8: torch.Tensor,
+    scale_weight: torch.Tensor,
+    weight_t_fp8: torch.Tensor,
+    scale_weight_t: torch.Tensor,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    return fp8_act_weight_gemm(input_2d.contiguous(), weight_fp8, scale_weight)
+
+
+@_fp8_linear_fwd.register_fake
+def _(input_2d, weight, weight_fp8, scale_weight, weight_t_fp8, scale_weight_t):
+    (M, K), N = input_2d.shape, weight.shape[0]
+    output = torch.empty((M, N), dtype=input_2d.dtype, device=input_2d.device)
+    input_t_fp8 = torch.empty((K, M), dtype=torch.float8_e4m3fn, device=input_2d.device)
+    size = ((K + 127) // 128, (M + 127) // 128)
+    scale_input_t = torch.empty(size, dtype=torch.float32, device=input_2d.device)
+    return output, input_t_fp8, scale_input_t
+
+
+@torch.library.custom_op("pith_train_amd::fp8_linear_bwd", mutates_args=())
+def _fp8_linear_bwd(
+    grad_output_2d: torch.Tensor,
+    weight_t_fp8: torch.Tensor,
+    scale_weight_t: torch.Tensor,
+    input_t_fp8: torch.Tensor,
+    scale_input_t: torch.Tensor,
+    K: int,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    return fp8_dgrad_wgrad(
+        grad_output_2d.contiguous(), weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t, K
+    )
+
+
+@_fp8_linear_bwd.register_fake
+def _(grad_output_2d, weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t, K):
+    M, N = grad_output_2d.shape
+    grad_input = torch.empty((M, K), dtype=grad_output_2d.dtype, device=grad_output_2d.device)
+    weight_grad = torch.empty((N, K), dtype=grad_output_2d.dtype, device=grad_output_2d.device)
+    return grad_input, weight_grad
+
+
+def _fp8_linear_setup_context(ctx, inputs, output):
+    input_2d, _, _, _, weight_t_fp8, scale_weight_t = inputs
+    _, input_t_fp8, scale_input_t = output
+    ctx.save_for_backward(weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t)
+    ctx.K = input_2d.shape[1]
+
+
+def _fp8_linear_backward(ctx, grad_output, grad_input_t_fp8, grad_scale_input_t):
+    weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t = ctx.saved_tensors
+    grad_input, weight_grad = _fp8_linear_bwd(
+        grad_output, weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t, ctx.K
+    )
+    return grad_input, weight_grad, None, None, None, None
+
+
+_fp8_linear_fwd.register_autograd(_fp8_linear_backward, setup_context=_fp8_linear_setup_context)
+
+
+class FP8Linear(nn.Linear):
+    """``nn.Linear`` whose three GEMMs run in FP8; the bf16 weight is quantised once per
+    ``FP8WeightCacheControl.version`` and reused across micro-batches."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self._wq_cache = None
+        self._wq_version: int = -1
+
+    def _get_quantized_weight(self):
+        if torch.compiler.is_compiling():
+            return fp8cast_blockwise_transpose(self.weight)
+        ver = FP8WeightCacheControl.version
+        if self._wq_version == ver and self._wq_cache is not None:
+            return self._wq_cache
+        result = fp8cast_blockwise_transpose(self.weight)
+        self._wq_cache = result
+        self._wq_version = ver
+        return result
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        if input.numel() == 0:
+            return torch.nn.functional.linear(input, self.weight, self.bias)
+        weight_fp8, scale_weight, weight_t_fp8, scale_weight_t = self._get_quantized_weight()
+        input_2d = input.flatten(0, -2)
+        output_2d, _, _ = _fp8_linear_fwd(
+            input_2d, self.weight, weight_fp8, scale_weight, weight_t_fp8, scale_weight_t
+        )
+        output = output_2d.view(*input.shape[:-1], self.weight.shape[0])
+        if self.bias is not None:
+            output = output + self.bias
+        return output

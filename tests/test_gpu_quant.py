@@ -1,0 +1,143 @@
+"""GPU parity: the six quantisers through the C-ABI vs the CPU oracle, bit for bit.
+
+Shapes follow the reference's own lists (tests/operators/test_deepgemm_quantize.py:50-61,
+111-122,169-182,229-240,305-315) plus ragged / strided / fp32 / extreme-magnitude cases.
+"""
+
+import pytest
+import torch
+
+from oracle import fp8 as Q
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from pith_train_amd.operators import deepgemm_quantize as D
+
+    return D
+
+
+def _mk(shape, seed, dtype=torch.bfloat16, spread=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g)
+    if spread:  # per-row magnitudes over many binades so many different scales occur
+        x = x * torch.exp2(torch.randint(-12, 12, (shape[0],) + (1,) * (len(shape) - 1), generator=g).float())
+    x = x.to(dtype)
+    x.view(-1)[0] = -0.0
+    return x
+
+
+def _eq(got, ref, what):
+    got = got.cpu()
+    assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert got.dtype == ref.dtype, f"{what}: dtype {got.dtype} vs {ref.dtype}"
+    if got.dtype == torch.float8_e4m3fn:
+        got, ref = got.view(torch.uint8), ref.view(torch.uint8)
+    bad = (got != ref).sum().item()
+    assert bad == 0, f"{what}: {bad} of {got.numel()} elements differ"
+
+
+ROWCOL = [(128, 128), (128, 256), (256, 256), (256, 512), (384, 384), (128, 300), (256, 7168), (128, 7), (1024, 2880)]
+
+
+@pytest.mark.parametrize("M,N", ROWCOL)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rowwise_colwise(M, N, dtype):
+    D = _ops()
+    x = _mk((M, N), M * 7 + N, dtype)
+    ref = Q.fp8cast_rowwise_colwise(x)
+    got = D.fp8cast_rowwise_colwise(x.cuda())
+    for g, r, w in zip(got, ref, ("tok_fp8", "tok_scale", "ch_fp8", "ch_scale")):
+        _eq(g, r, w)
+    got_t = D.fp8cast_rowwise_colwise_t(x.cuda())
+    _eq(got_t[0], ref[0], "tok_fp8")
+    _eq(got_t[1], ref[1], "tok_scale")
+    _eq(got_t[2], ref[2].view(torch.uint8).T.contiguous().view(torch.float8_e4m3fn), "ch_t_fp8")
+    _eq(got_t[3], ref[3], "ch_scale")
+
+
+def test_rowwise_colwise_all_zero_and_strided():
+    D = _ops()
+    z = torch.zeros((128, 256), dtype=torch.bfloat16)
+    tok, tok_s, ch, ch_s = D.fp8cast_rowwise_colwise(z.cuda())
+    assert (tok.view(torch.uint8) == 0).all() and (ch.view(torch.uint8) == 0).all()
+    assert (tok_s == 2.0**-22).all() and (ch_s == 2.0**-22).all()
+    big = _mk((256, 512), 3)
+    view = big[:, 128:384]  # row stride 512, 256 columns
+    ref = Q.fp8cast_rowwise_colwise(view.contiguous())
+    got = D.fp8cast_rowwise_colwise(big.cuda()[:, 128:384])
+    for g, r, w in zip(got, ref, ("tok_fp8", "tok_scale", "ch_fp8", "ch_scale")):
+        _eq(g, r, w)
+
+
+def test_rowwise_kmajor():
+    D = _ops()
+    offs = torch.tensor([128, 128, 512, 640, 1024], dtype=torch.int32)
+    x = _mk((1024, 200), 17)
+    ref = Q.fp8cast_rowwise_kmajor(x, offs)
+    got = D.fp8cast_rowwise_kmajor(x.cuda(), offs.cuda())
+    for g, r, w in zip(got, ref, ("tok_fp8", "tok_scale", "kmajor_fp8", "kmajor_scale")):
+        _eq(g, r, w)
+
+
+TRANS = [(128, 128), (128, 256), (256, 256), (64, 256), (7, 300), (1, 128), (256, 7168), (64, 64), (300, 130), (4096, 512)]
+
+
+@pytest.mark.parametrize("M,N", TRANS)
+def test_rowwise_transpose(M, N):
+    D = _ops()
+    x = _mk((M, N), M * 11 + N)
+    ref = Q.fp8cast_rowwise_transpose(x)
+    got = D.fp8cast_rowwise_transpose(x.cuda())
+    for g, r, w in zip(got, ref, ("tok_fp8", "tok_scale", "t_fp8", "t_scale")):
+        _eq(g, r, w)
+
+
+@pytest.mark.parametrize("M,K", TRANS)
+def test_rowwise_blockwise_transpose(M, K):
+    D = _ops()
+    x = _mk((M, K), M * 13 + K)
+    ref = Q.fp8cast_rowwise_blockwise_transpose(x)
+    got = D.fp8cast_rowwise_blockwise_transpose(x.cuda())
+    for g, r, w in zip(got, ref, ("tok_fp8", "tok_scale", "blk_t_fp8", "blk_t_scale")):
+        _eq(g, r, w)
+
+
+@pytest.mark.parametrize("M,K", TRANS + [(2880, 2880)])
+def test_blockwise_transpose(M, K):
+    D = _ops()
+    x = _mk((M, K), M * 17 + K)
+    ref = Q.fp8cast_blockwise_transpose(x)
+    got = D.fp8cast_blockwise_transpose(x.cuda())
+    for g, r, w in zip(got, ref, ("fp8", "scale", "fp8_t", "scale_t")):
+        _eq(g, r, w)
+    assert torch.equal(got[1], got[3].T)
+
+
+@pytest.mark.parametrize("G,N,K", [(1, 128, 128), (4, 256, 128), (3, 200, 300), (8, 512, 256), (2, 2880, 320)])
+def test_blockwise_transpose_batched(G, N, K):
+    D = _ops()
+    g = torch.Generator().manual_seed(G * 100 + N + K)
+    w = (torch.randn((G, N, K), generator=g) * 0.02).bfloat16()
+    ref = Q.fp8cast_blockwise_transpose_batched(w)
+    got = D.fp8cast_blockwise_transpose_batched(w.cuda())
+    for a, r, name in zip(got, ref, ("fp8", "scale", "fp8_t", "scale_t")):
+        _eq(a, r, name)
+    assert torch.equal(got[1], got[3].transpose(1, 2))
+
+
+def test_every_bf16_value_roundtrips_like_the_oracle():
+    """All 65280 finite bf16 bit patterns in one tensor (rows sorted by magnitude so scales vary)."""
+    D = _ops()
+    bits = torch.arange(0, 1 << 16, dtype=torch.int32).to(torch.int16)
+    x = bits.view(torch.bfloat16)
+    x = x[torch.isfinite(x.float())]
+    x = x[torch.argsort(x.float().abs(), stable=True)]
+    n = (x.numel() // (128 * 128)) * 128 * 128
+    x = x[-n:].reshape(-1, 128).contiguous()
+    x = x[: (x.shape[0] // 128) * 128]
+    ref = Q.fp8cast_rowwise_colwise(x)
+    got = D.fp8cast_rowwise_colwise(x.cuda())
+    for g, r, w in zip(got, ref, ("tok_fp8", "tok_scale", "ch_fp8", "ch_scale")):
+        _eq(g, r, w)
