@@ -1,0 +1,264 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 grouped-expert path on one MI355X.
+
+One "step" = one full MoE expert layer (stage 3) forward + backward over one batch of synthetic
+tokens resident in HBM: weight quantisation (every step - nothing is cached across steps), token
+scatter, gate/up grouped GEMM, SwiGLU, down grouped GEMM, unpermute, and the whole backward
+(dgrad + wgrad GEMMs, epilogue backward, gathers).
+
+Prints ONE JSON line.  ``value`` is algorithmic GEMM TFLOP/s of the whole step (padding rows not
+counted); ``roofline`` describes the dominant kernel (the FP8 MFMA GEMM) from HIP-event timings
+taken around every GEMM launch inside the timed region; ``cpu_baseline`` is the CPU oracle of the
+same layer (the reference's pure-PyTorch BF16 grouped-linear semantics) on a bounded sample.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+FP8_DENSE_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (kind, hidden, intermediate, experts, top_k, tokens, zipf)
+    "qwen3-30b-a3b-moe": ("fused", 2048, 768, 128, 8, 8192, None),
+    "toy": ("split", 256, 512, 8, 2, 1024, None),
+    "dsv2-lite-moe": ("split", 2048, 1408, 64, 6, 8192, 1.2),
+    "gpt-oss-20b-moe": ("gpt_oss", 2880, 2880, 32, 4, 16384, None),
+}
+
+
+def make_inputs(kind, H, I, E, k, T, zipf, seed=0):
+    import torch
+
+    from oracle import moe as OM
+
+    ids = OM.make_routing(T, E, k, seed=seed, zipf_s=zipf)
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((T, H), generator=g).bfloat16()
+    dy = torch.randn((T * k, H), generator=g).bfloat16()
+    r = lambda *s: (torch.randn(s, generator=g) * 0.02).bfloat16()  # noqa: E731
+    if kind == "split":
+        w = {"gate_proj": r(E, I, H), "up_proj": r(E, I, H), "down_proj": r(E, H, I)}
+    elif kind == "fused":
+        w = {"gate_up_proj": r(E, 2 * I, H), "down_proj": r(E, H, I)}
+    else:
+        w = {"gate_up_proj": r(E, 2 * I, H), "gate_up_proj_bias": r(E, 2 * I), "down_proj": r(E, H, I),
+             "down_proj_bias": r(E, H)}
+    return ids, x, dy, w
+
+
+def build_module(kind, H, I, E, w):
+    import torch
+
+    from pith_train_amd.modules import experts as X
+
+    if kind == "split":
+        mod = X.Qwen3MoeExperts(H, I, E)
+    elif kind == "fused":
+        mod = X.Qwen35MoeExperts(H, I, E)
+    else:
+        mod = X.GptOssExperts(H, I, E)
+    mod = mod.cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        for n, v in w.items():
+            p = getattr(mod, n)
+            (p if kind == "gpt_oss" else p.weight).copy_(v.cuda())
+    return mod
+
+
+class GemmTimer:
+    """HIP events (on the stream the kernels are launched on) around every GEMM entry point."""
+
+    NAMES = ("pt_gemm_m_grouped_nt", "pt_gemm_k_grouped_wgrad", "pt_gemm_nt_dense")
+
+    def __init__(self):
+        self.records = []
+        self.enabled = False
+
+    def install(self):
+        import torch
+
+        from pith_train_amd import _lib
+
+        orig = _lib.call
+        timer = self
+
+        def call(name, *args):
+            if timer.enabled and name in GemmTimer.NAMES:
+                a = torch.cuda.Event(enable_timing=True)
+                b = torch.cuda.Event(enable_timing=True)
+                a.record()
+                orig(name, *args)
+                b.record()
+                timer.records.append((name, a, b))
+            else:
+                orig(name, *args)
+
+        _lib.call = call
+        # modules imported `_lib` (the module), so they see the patched attribute
+        return self
+
+    def summary(self):
+        out = {}
+        for name, a, b in self.records:
+            d = out.setdefault(name, [0.0, 0])
+            d[0] += a.elapsed_time(b)
+            d[1] += 1
+        return {k: {"ms_total": v[0], "launches": v[1]} for k, v in out.items()}
+
+
+def cpu_baseline(kind, H, I, E, k, T, zipf, budget_s=12.0):
+    """The CPU oracle of the same layer on the same seeded inputs: the BF16 grouped-linear
+    semantics (the reference's pure-PyTorch path), forward + backward, all host cores given to
+    torch.  The whole workload is repeated until about ``budget_s`` seconds have been spent."""
+    import torch
+
+    from oracle import moe as OM
+
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    ids, x, dy, w = make_inputs(kind, H, I, E, k, T, zipf, seed=0)
+    tokens = x.unsqueeze(1).expand(-1, k, -1).reshape(-1, H).contiguous()
+    eidx = ids.reshape(-1)
+    flops = OM.gemm_flops(T * k, H, I)
+    OM.moe_layer_fwd_bwd(tokens[:512], eidx[:512], w, dy[:512], E, kind=kind, fp8=False)  # warm
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        OM.moe_layer_fwd_bwd(tokens, eidx, w, dy, E, kind=kind, fp8=False)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or reps >= 20:
+            break
+    sec = el / reps
+    return {
+        "value": flops / sec / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"full workload ({T * k} routed rows, {E} experts), bf16 grouped-linear oracle fwd+bwd on the host, "
+                  f"{reps} rep(s), {sec:.2f} s each",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="qwen3-30b-a3b-moe", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cached-weights", action="store_true",
+                    help="also report a step time with the FP8 weight cache kept across steps")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU's share of the expert path; run with --gpus 1 "
+              "(no collectives or multi-GPU sharding are part of it).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from oracle import moe as OM
+    from pith_train_amd import _lib
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules.experts import forward_stage3
+
+    _lib.load()  # fail loudly if the HIP library is missing
+    kind, H, I, E, k, T, zipf = WORKLOADS[args.workload]
+    ids, x, dy, w = make_inputs(kind, H, I, E, k, T, zipf)
+    mod = build_module(kind, H, I, E, w)
+    params = [p for p in mod.parameters()]
+    tokens = x.cuda().unsqueeze(1).expand(-1, k, -1).reshape(-1, H).contiguous()
+    eidx = ids.reshape(-1).cuda()
+    dyc = dy.cuda()
+    rows = T * k
+    flops = OM.gemm_flops(rows, H, I)
+    timer = GemmTimer().install()
+
+    def step(bump=True):
+        if bump:
+            FP8WeightCacheControl.step()  # re-quantise the weights: nothing carried across steps
+        for p in params:
+            p.grad = None
+        tok = tokens.detach().requires_grad_(True)
+        out = forward_stage3(mod, tok, eidx, E)
+        out.backward(dyc)
+        return tok.grad
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer.enabled = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    timer.enabled = False
+    ms = elapsed / args.steps * 1e3
+
+    gs = timer.summary()
+    gemm_ms = sum(v["ms_total"] for v in gs.values())
+    gemm_launches = sum(v["launches"] for v in gs.values())
+    achieved = flops * args.steps / (gemm_ms * 1e-3) / 1e12 if gemm_ms > 0 else 0.0
+
+    extra = {}
+    if args.cached_weights:
+        for _ in range(2):
+            step(bump=False)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            step(bump=False)
+        torch.cuda.synchronize()
+        extra["ms_per_step_weights_cached"] = (time.perf_counter() - t1) / args.steps * 1e3
+
+    result = {
+        "metric": "MoE-layer fwd+bwd TFLOP/s (FP8 grouped-expert path, Qwen3-30B-A3B shape, 1 GPU)"
+        if args.workload == "qwen3-30b-a3b-moe" else f"MoE-layer fwd+bwd TFLOP/s ({args.workload})",
+        "value": flops / (ms * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3 (fp32 accumulate, bf16 in/out)",
+        "data": "synthetic (seed 0: x~N(0,1) bf16, weights~N(0,0.02), grad~N(0,1), router logits~N(0,1) softmax top-k)",
+        "config": {
+            "workload": args.workload, "kind": kind, "hidden": H, "moe_intermediate": I, "experts": E,
+            "top_k": k, "tokens": T, "routed_rows": rows, "algorithmic_gemm_tflop_per_step": flops / 1e12,
+            "weight_quant_in_step": True,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "kernel": "fp8_gemm_nt_kernel (all grouped GEMM launches of the step: fwd, dgrad, wgrad)",
+            "achieved": achieved,
+            "peak": FP8_DENSE_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / FP8_DENSE_PEAK_TFLOPS,
+            "traffic": None,
+            "launches_per_step": gemm_launches / max(args.steps, 1),
+            "gemm_ms_per_step": gemm_ms / max(args.steps, 1),
+            "per_entry_point_ms_per_step": {k2: v["ms_total"] / args.steps for k2, v in gs.items()},
+        },
+        **extra,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(kind, H, I, E, k, T, zipf)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -29,6 +29,14 @@ ARCH_MAJOR = 9
 def _fp8_gemm_nt(a_fp8, a_scale, b_fp8, b_scale, m: int, n: int, device, dtype) -> torch.Tensor:
     """out[m, n] = a @ b.T; a: 1x128 scales, b: 128x128 scales."""
     k = a_fp8.shape[1]
+    if k % 16:
+        # The kernels fetch 16-byte chunks along the reduction dimension.  A ragged length (a
+        # wgrad over a token count that is not a multiple of 16) is zero-padded; the padding stays
+        # inside the last 128-block, so the scale grids are unchanged.
+        pad = 16 - k % 16
+        a_fp8 = torch.nn.functional.pad(a_fp8.view(torch.uint8), (0, pad)).view(torch.float8_e4m3fn)
+        b_fp8 = torch.nn.functional.pad(b_fp8.view(torch.uint8), (0, pad)).view(torch.float8_e4m3fn)
+        k += pad
     out_dtype = dtype if dtype in (torch.bfloat16, torch.float32) else torch.float32
     out = torch.empty((m, n), device=device, dtype=out_dtype)
     _lib.call(

@@ -138,7 +138,8 @@ def test_k_grouped_wgrad(sizes, N, K, accumulate):
         diff = (out.cpu().float() - expect.float()).abs()
         # one bf16 ulp of slack: the kernel's fp32 sum may round to the neighbouring bf16 value
         # (relative to the operands, not to the possibly cancelling result)
-        ulp = (old.float().abs() + ref.float().abs()) * 2.0**-6 + 1e-6
+        # plus the fp32 accumulation-order noise of the sum itself (matters where it cancels to ~0)
+        ulp = (old.float().abs() + ref.float().abs()) * 2.0**-6 + 1e-3 * ref.float().pow(2).mean().sqrt()
         assert (diff <= ulp).all(), diff.max().item()
         old32 = old.float()
         out32 = old32.clone().cuda()

@@ -1,0 +1,239 @@
+"""GPU parity of the composed path: expert modules, stage 3, dense FP8 linear, deferred wgrad.
+
+Oracle: ``oracle.moe`` / ``oracle.gemm`` (float64 accumulation over bit-identical FP8 operands).
+Intermediate activations are rounded to bf16 and re-quantised, so a last-bit difference in one
+GEMM output can move a later FP8 byte; the end-to-end bound is therefore the similarity metric
+of the reference's FP8 tests (``calc_diff < 1e-3``,
+tests/test_deepgemm_fp8_linear_correctness.py:14) plus max |err| <= 5e-2 x max |ref| (one FP8 step is
+2**-4 of the element).
+"""
+
+import pytest
+import torch
+
+from oracle import gemm as G
+from oracle import moe as OM
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(got, ref, what, rel=5e-2, diff=1e-3):
+    got, ref = got.detach().float().cpu().double(), ref.double()
+    assert got.shape == ref.shape, f"{what}: {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert torch.isfinite(got).all(), what
+    d = G.calc_diff(got, ref)
+    worst = (got - ref).abs().max().item()
+    scale = ref.abs().max().item()
+    assert d < diff, f"{what}: calc_diff {d:.3e}"
+    assert worst <= rel * scale + 1e-30, f"{what}: max err {worst:.3e} vs max |ref| {scale:.3e}"
+
+
+def _weights(kind, E, H, I, seed):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: (torch.randn(s, generator=g) * 0.02).bfloat16()  # noqa: E731
+    if kind == "split":
+        return {"gate_proj": r(E, I, H), "up_proj": r(E, I, H), "down_proj": r(E, H, I)}
+    if kind == "fused":
+        return {"gate_up_proj": r(E, 2 * I, H), "down_proj": r(E, H, I)}
+    return {"gate_up_proj": r(E, 2 * I, H), "gate_up_proj_bias": r(E, 2 * I), "down_proj": r(E, H, I),
+            "down_proj_bias": r(E, H)}
+
+
+def _build(kind, E, H, I, w):
+    from pith_train_amd.modules import experts as X
+
+    if kind == "split":
+        mod = X.Qwen3MoeExperts(H, I, E)
+        params = {"gate_proj": mod.gate_proj.weight, "up_proj": mod.up_proj.weight, "down_proj": mod.down_proj.weight}
+    elif kind == "fused":
+        mod = X.Qwen35MoeExperts(H, I, E)
+        params = {"gate_up_proj": mod.gate_up_proj.weight, "down_proj": mod.down_proj.weight}
+    else:
+        mod = X.GptOssExperts(H, I, E)
+        params = {k: getattr(mod, k) for k in w}
+    mod = mod.cuda().to(torch.bfloat16)
+    params = {k: (getattr(mod, k) if kind == "gpt_oss" else getattr(mod, k).weight) for k in params}
+    with torch.no_grad():
+        for k, p in params.items():
+            p.copy_(w[k].cuda())
+    return mod, params
+
+
+CASES = [
+    ("split", 8, 256, 128, 1024, 2, None),        # toy: 8 experts, top-2
+    ("fused", 16, 512, 256, 512, 4, None),
+    ("gpt_oss", 4, 384, 384, 300, 2, None),       # 384 = 3 x 128; biases, clamped SwiGLU
+    ("gpt_oss", 4, 320, 192, 256, 2, None),       # K, N not multiples of 128
+    ("split", 16, 256, 128, 700, 3, 1.2),         # Zipf skew: empty and crowded experts
+]
+
+
+@pytest.mark.parametrize("kind,E,H,I,T,k,zipf", CASES)
+def test_stage3_forward_backward(kind, E, H, I, T, k, zipf):
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules.experts import forward_stage3
+
+    ids = OM.make_routing(T, E, k, seed=0, zipf_s=zipf)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn((T, H), generator=g).bfloat16()
+    tokens = x.unsqueeze(1).expand(-1, k, -1).reshape(-1, H).contiguous()
+    expert_idxs = ids.reshape(-1)
+    dy = torch.randn((T * k, H), generator=g).bfloat16()
+    w = _weights(kind, E, H, I, 2)
+    ref = OM.moe_layer_fwd_bwd(tokens, expert_idxs, w, dy, E, kind=kind, fp8=True, accum=torch.float64)
+
+    mod, params = _build(kind, E, H, I, w)
+    FP8WeightCacheControl.step()
+    tok = tokens.cuda().requires_grad_(True)
+    out = forward_stage3(mod, tok, expert_idxs.cuda(), E)
+    _close(out, ref["out"], "out")
+    out.backward(dy.cuda())
+    _close(tok.grad, ref["grad_tokens"], "grad_tokens")
+    for name, p in params.items():
+        assert p.grad is not None and p.grad.dtype == torch.bfloat16, name
+        _close(p.grad, ref[name], name)
+
+
+def test_stage3_with_dedup_expand_fused_and_unfused():
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules.experts import forward_stage3
+
+    E, H, I, U, R = 8, 256, 128, 300, 1000
+    g = torch.Generator().manual_seed(7)
+    uniq = torch.randn((U, H), generator=g).bfloat16()
+    expand = torch.randint(0, U, (R,), generator=g)
+    eidx = torch.randint(0, E, (R,), generator=g)
+    dy = torch.randn((R, H), generator=g).bfloat16()
+    w = _weights("split", E, H, I, 3)
+    ref = OM.moe_layer_fwd_bwd(uniq, eidx, w, dy, E, kind="split", fp8=True, expand_idx=expand, accum=torch.float64)
+    mod, params = _build("split", E, H, I, w)
+    grads = []
+    for fuse in (True, False):
+        FP8WeightCacheControl.step()
+        for p in params.values():
+            p.grad = None
+        t = uniq.cuda().requires_grad_(True)
+        out = forward_stage3(mod, t, eidx.cuda(), E, expand_idx=expand.cuda(), fuse_expand=fuse)
+        _close(out, ref["out"], f"out fuse={fuse}")
+        out.backward(dy.cuda())
+        _close(t.grad, ref["grad_tokens"], f"grad_tokens fuse={fuse}")
+        grads.append(t.grad.clone())
+    assert torch.equal(grads[0], grads[1])
+
+
+def test_grouped_linear_defers_wgrad_and_accumulates():
+    """WeightGradStore contract (grouped_linear.py:223-234; test file :239-290 of the reference)."""
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl, WeightGradStore
+    from pith_train_amd.operators.grouped_linear import FP8GroupedLinear, GroupedLinear
+    from pith_train_amd.operators.token_scatter import scatter_for_grouped_gemm
+
+    E, K, N = 4, 128, 256
+    fp8 = FP8GroupedLinear(E, K, N).cuda().to(torch.bfloat16)
+    bf16 = GroupedLinear(E, K, N).cuda().to(torch.bfloat16)
+    torch.manual_seed(0)
+    torch.nn.init.normal_(fp8.weight, std=0.02)
+    bf16.weight.data.copy_(fp8.weight.data)
+    x = torch.randn(64, K, device="cuda", dtype=torch.bfloat16)
+    e = torch.randint(0, E, (64,), device="cuda")
+    xs, _, offs, ks, kst = scatter_for_grouped_gemm(x, e, E)
+    grad = torch.randn(xs.shape[0], N, device="cuda", dtype=torch.bfloat16)
+
+    FP8WeightCacheControl.step()
+    a = xs.detach().clone().requires_grad_(True)
+    fp8(a, offs, ks=ks, ks_tensor=kst).backward(grad)
+    direct = fp8.weight.grad.clone()
+    b = xs.detach().clone().requires_grad_(True)
+    bf16(b, offs).backward(grad)
+    assert G.calc_diff(direct.cpu(), bf16.weight.grad.cpu()) < 1e-3
+    assert G.calc_diff(a.grad.cpu(), b.grad.cpu()) < 1e-3
+
+    fp8.weight.grad = None
+    WeightGradStore.clear()
+    WeightGradStore.enabled = True
+    try:
+        c = xs.detach().clone().requires_grad_(True)
+        fp8(c, offs, ks=ks, ks_tensor=kst).backward(grad)
+        assert fp8.weight.grad is None and len(WeightGradStore.cache) == 1
+        WeightGradStore.flush()
+        WeightGradStore.pop()
+    finally:
+        WeightGradStore.enabled = False
+        WeightGradStore.clear()
+    assert torch.equal(fp8.weight.grad, direct)
+    # second backward accumulates into the existing bf16 grad
+    d = xs.detach().clone().requires_grad_(True)
+    fp8(d, offs, ks=ks, ks_tensor=kst).backward(grad)
+    assert torch.equal(fp8.weight.grad, (direct.float() + direct.float()).bfloat16())
+
+
+def test_weight_cache_versioning_and_empty_input():
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.operators.grouped_linear import FP8GroupedLinear
+    from pith_train_amd.operators.linear import FP8Linear
+
+    gl = FP8GroupedLinear(2, 128, 128).cuda().to(torch.bfloat16)
+    torch.nn.init.normal_(gl.weight, std=0.02)
+    FP8WeightCacheControl.step()
+    q1 = gl._get_quantized_weight()
+    assert gl._get_quantized_weight() is q1
+    FP8WeightCacheControl.step()
+    assert gl._get_quantized_weight() is not q1
+    FP8WeightCacheControl.clear(gl)
+    assert gl._wq_cache is None
+    out = gl(torch.empty(0, 128, device="cuda", dtype=torch.bfloat16, requires_grad=True),
+             torch.empty(0, dtype=torch.int32, device="cuda"), [], None)
+    assert out.shape == (0, 128) and out.grad_fn is not None
+    lin = FP8Linear(128, 64, bias=True).cuda().to(torch.bfloat16)
+    o = lin(torch.empty(0, 128, device="cuda", dtype=torch.bfloat16))
+    assert o.shape == (0, 64)
+
+
+@pytest.mark.parametrize("M,K,N,bias", [(256, 256, 512, False), (300, 384, 200, True), (4096, 2048, 512, False)])
+def test_fp8_linear_forward_backward(M, K, N, bias):
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.operators.linear import FP8Linear
+
+    g = torch.Generator().manual_seed(M)
+    x = torch.randn((M, K), generator=g).bfloat16()
+    w = (torch.randn((N, K), generator=g) * 0.02).bfloat16()
+    dy = torch.randn((M, N), generator=g).bfloat16()
+    y_ref, saved = G.fp8_linear_forward(x, w)
+    gi_ref, gw_ref = G.fp8_linear_backward(dy, saved)
+    lin = FP8Linear(K, N, bias=bias).cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(w.cuda())
+        if bias:
+            lin.bias.normal_(std=0.02)
+    FP8WeightCacheControl.step()
+    xc = x.cuda().view(2, M // 2, K).requires_grad_(True)
+    y = lin(xc)
+    assert y.shape == (2, M // 2, N)
+    ref = y_ref if not bias else (y_ref + lin.bias.detach().cpu())
+    _close(y.reshape(M, N), ref, "y")
+    y.backward(dy.cuda().view(2, M // 2, N))
+    _close(xc.grad.reshape(M, K), gi_ref, "grad_input")
+    _close(lin.weight.grad, gw_ref, "weight_grad")
+    if bias:
+        _close(lin.bias.grad, dy.float().sum(0), "bias_grad", rel=2e-2)
+
+
+def test_dense_mlp_and_bf16_switch():
+    from pith_train_amd.modules import experts as X
+    from pith_train_amd.modules import training
+
+    mlp = X.DeepSeekV2MLP(256, 384).cuda().to(torch.bfloat16)
+    for p in mlp.parameters():
+        torch.nn.init.normal_(p, std=0.02)
+    x = torch.randn(512, 256, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    y = mlp(x)
+    ref = torch.nn.functional.linear(
+        torch.nn.functional.silu(x @ mlp.gate_proj.weight.T) * (x @ mlp.up_proj.weight.T), mlp.down_proj.weight)
+    # three chained FP8 GEMMs against pure bf16: looser than the single-layer 1e-3
+    assert G.calc_diff(y.detach().cpu(), ref.detach().cpu()) < 5e-3
+    y.sum().backward()
+    assert x.grad is not None and mlp.gate_proj.weight.grad is not None
+    try:
+        training.setup(False)
+        assert training.Linear is torch.nn.Linear and training.GroupedLinear.__name__ == "GroupedLinear"
+    finally:
+        training.setup(True)
