@@ -15,28 +15,13 @@
 // ds_read_b128 fragment reads are spread over the banks.  Per step a wave reads all of its
 // fragments, then the next tile's loads are issued, then the MFMAs run while those loads land.
 #include "common.h"
+#include "gemm_args.h"
+#include <stdlib.h>
 
 namespace pt {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-
-enum { GEMM_DENSE = 0, GEMM_M_GROUPED = 1, GEMM_K_GROUPED = 2 };
-
-struct GemmArgs {
-  const uint8_t* a; int64_t lda;          // [rows_a, red] bytes
-  const uint8_t* b; int64_t ldb;          // [rows_b, red] bytes
-  const float* sa; int64_t sa_rs, sa_ks; int sa_shift;  // scale(row,kb) = sa[(row>>shift)*rs + kb*ks]
-  const float* sb; int64_t sb_rs, sb_ks; int sb_shift;
-  void* out; int64_t ldo;                 // elements
-  int out_dtype; int accumulate;
-  int64_t rows_a, rows_b, red;            // output is rows_a x rows_b; red = reduction length (dense / m-grouped)
-  const int32_t* offs; int G;
-  int mode;
-  int64_t b_stride_g, sb_stride_g, out_stride_g;
-  int tiles_a, tiles_b;                   // tile counts along rows_a / rows_b
-  int64_t total_tiles;
-};
 
 __device__ __attribute__((aligned(16))) uint32_t g_zero_chunk[4] = {0, 0, 0, 0};
 
@@ -275,6 +260,30 @@ static int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   return check_launch("fp8_gemm_nt_kernel");
 }
 
+// PT_GEMM_IMPL selects the kernel for experiments: "tile" = one tile per workgroup (128x128),
+// "p0" / "p1" / "p2" = persistent kernel variants.  Default: persistent 256x256.
+static int gemm_impl() {
+  static int impl = -2;
+  if (impl == -2) {
+    const char* e = getenv("PT_GEMM_IMPL");
+    if (!e || !*e) impl = 0;
+    else if (e[0] == 't') impl = -1;
+    else if (e[0] == 'p') impl = atoi(e + 1);
+    else impl = 0;
+  }
+  return impl;
+}
+
+static int dispatch_gemm(const GemmArgs& g, hipStream_t stream) {
+  const int impl = gemm_impl();
+  // the persistent kernel addresses operands through 32-bit buffer offsets
+  const int64_t lim = (1ll << 31) - 1;
+  const bool fits = g.a_bytes < lim && g.b_bytes < lim && g.sa_bytes < lim && g.sb_bytes < lim && g.rows_a < lim &&
+                    g.rows_b < lim && g.red < lim;
+  if (impl < 0 || !fits) return launch_gemm<128, 128, 2, 2>(g, stream);
+  return launch_gemm_persistent(g, impl, stream);
+}
+
 }  // namespace pt
 
 using namespace pt;
@@ -295,9 +304,10 @@ extern "C" int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const v
   g.sb = b_scale; g.sb_rs = KB; g.sb_ks = 1; g.sb_shift = 7;
   g.out = out; g.ldo = N; g.out_dtype = out_dtype; g.accumulate = 0;
   g.rows_a = M; g.rows_b = N; g.red = K; g.mode = GEMM_DENSE;
+  g.a_bytes = M * K; g.b_bytes = N * K; g.sa_bytes = M * KB * 4; g.sb_bytes = cdiv(N, 128) * KB * 4;
   g.tiles_a = (int)cdiv(M, 128); g.tiles_b = (int)cdiv(N, 128);
   g.total_tiles = (int64_t)g.tiles_a * g.tiles_b;
-  return launch_gemm<128, 128, 2, 2>(g, (hipStream_t)stream);
+  return dispatch_gemm(g, (hipStream_t)stream);
 }
 
 extern "C" int pt_gemm_m_grouped_nt(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
@@ -318,9 +328,10 @@ extern "C" int pt_gemm_m_grouped_nt(const void* a_fp8, const float* a_scale, con
   g.out = out; g.ldo = N; g.out_dtype = out_dtype; g.accumulate = 0;
   g.rows_a = M; g.rows_b = N; g.red = K; g.mode = GEMM_M_GROUPED; g.offs = offs; g.G = G;
   g.b_stride_g = N * K; g.sb_stride_g = NB * KB;
+  g.a_bytes = M * K; g.b_bytes = N * K; g.sa_bytes = M * KB * 4; g.sb_bytes = NB * KB * 4;
   g.tiles_a = (int)(M / 128); g.tiles_b = (int)NB;
   g.total_tiles = (int64_t)g.tiles_a * g.tiles_b;
-  return launch_gemm<128, 128, 2, 2>(g, (hipStream_t)stream);
+  return dispatch_gemm(g, (hipStream_t)stream);
 }
 
 extern "C" int pt_gemm_k_grouped_wgrad(const void* dy_t_fp8, const float* dy_scale, const void* x_t_fp8, const float* x_scale,
@@ -340,7 +351,8 @@ extern "C" int pt_gemm_k_grouped_wgrad(const void* dy_t_fp8, const float* dy_sca
   g.out = out; g.ldo = K; g.out_dtype = out_dtype; g.accumulate = accumulate;
   g.rows_a = N; g.rows_b = K; g.red = M; g.mode = GEMM_K_GROUPED; g.offs = offs; g.G = G;
   g.out_stride_g = N * K;
+  g.a_bytes = N * M; g.b_bytes = K * M; g.sa_bytes = (M / 128) * N * 4; g.sb_bytes = (M / 128) * K * 4;
   g.tiles_a = (int)cdiv(N, 128); g.tiles_b = (int)cdiv(K, 128);
   g.total_tiles = (int64_t)g.tiles_a * g.tiles_b * G;
-  return launch_gemm<128, 128, 2, 2>(g, (hipStream_t)stream);
+  return dispatch_gemm(g, (hipStream_t)stream);
 }

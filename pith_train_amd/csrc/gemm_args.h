@@ -1,0 +1,29 @@
+// Argument block shared by the FP8 GEMM kernels.
+#pragma once
+#include "common.h"
+
+namespace pt {
+
+enum { GEMM_DENSE = 0, GEMM_M_GROUPED = 1, GEMM_K_GROUPED = 2 };
+
+struct GemmArgs {
+  const uint8_t* a; int64_t lda;          // [rows_a, red] bytes
+  const uint8_t* b; int64_t ldb;          // [rows_b, red] bytes
+  const float* sa; int64_t sa_rs, sa_ks; int sa_shift;  // scale(row,kb) = sa[(row>>shift)*rs + kb*ks]
+  const float* sb; int64_t sb_rs, sb_ks; int sb_shift;
+  void* out; int64_t ldo;                 // elements
+  int out_dtype; int accumulate;
+  int64_t rows_a, rows_b, red;            // output is rows_a x rows_b; red = reduction length (dense / m-grouped)
+  const int32_t* offs; int G;
+  int mode;
+  int64_t b_stride_g, sb_stride_g, out_stride_g;
+  int tiles_a, tiles_b;                   // tile counts along rows_a / rows_b
+  int64_t a_bytes, b_bytes, sa_bytes, sb_bytes;  // extents of a, one group of b, and their scale arrays
+  int64_t total_tiles;
+};
+
+
+// persistent-kernel launcher (gemm_persistent.hip); variant selects the tile shape
+int launch_gemm_persistent(const GemmArgs& a, int variant, hipStream_t stream);
+
+}  // namespace pt
