@@ -304,7 +304,7 @@ extern "C" int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const v
   g.sb = b_scale; g.sb_rs = KB; g.sb_ks = 1; g.sb_shift = 7;
   g.out = out; g.ldo = N; g.out_dtype = out_dtype; g.accumulate = 0;
   g.rows_a = M; g.rows_b = N; g.red = K; g.mode = GEMM_DENSE;
-  g.a_bytes = M * K; g.b_bytes = N * K; g.sa_bytes = M * KB * 4; g.sb_bytes = cdiv(N, 128) * KB * 4;
+  g.a_bytes = M * g.lda; g.b_bytes = N * g.ldb; g.sa_bytes = M * KB * 4; g.sb_bytes = cdiv(N, 128) * KB * 4;
   g.tiles_a = (int)cdiv(M, 128); g.tiles_b = (int)cdiv(N, 128);
   g.total_tiles = (int64_t)g.tiles_a * g.tiles_b;
   return dispatch_gemm(g, (hipStream_t)stream);

@@ -20,6 +20,7 @@ struct GemmArgs {
   int tiles_a, tiles_b;                   // tile counts along rows_a / rows_b
   int64_t a_bytes, b_bytes, sa_bytes, sb_bytes;  // extents of a, one group of b, and their scale arrays
   int64_t total_tiles;
+  int pf_dist;                            // L2 prefetch distance in 128-blocks beyond the LDS ring
 };
 
 

@@ -17,6 +17,7 @@
 //    XCDs, each with its own L2) and tiles that share a b-tile are adjacent.
 #include "common.h"
 #include "gemm_args.h"
+#include <stdlib.h>
 
 namespace pt {
 
@@ -44,11 +45,15 @@ __device__ __forceinline__ v4i make_rsrc(const void* base, uint32_t bytes) {
 // Direct-to-LDS buffer loads: address = base + voff (per lane) + soff (uniform); lane l's data lands
 // at lds_off + 16*l (dwordx4) or lds_off + 4*l (dword).  lds_off is a wave-uniform LDS byte address.
 __device__ __forceinline__ void dma16(v4i rsrc, uint32_t voff, uint32_t soff, uint32_t lds_off) {
+  soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);  // uniform by construction; pin them to SGPRs
+  lds_off = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_off);
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff),
                "s"(lds_off)
                : "memory");
 }
 __device__ __forceinline__ void dma4(v4i rsrc, uint32_t voff, uint32_t soff, uint32_t lds_off) {
+  soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
+  lds_off = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_off);
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff),
                "s"(lds_off)
                : "memory");
@@ -113,20 +118,21 @@ struct Tile {
   int a_row0, b_row0, a_lim, b_lim, k_begin, k_len, kb0, g;
 };
 
-template <int MODE, int BM, int BN, int WGM, int WGN>
+template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC>
 __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kernel(GemmArgs p) {
   constexpr int NW = WGM * WGN;
   constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int BK = 64;                       // reduction depth of one pipeline stage (one MFMA step)
-  constexpr int NS = 4;                        // stages in the LDS ring; NS-1 are in flight ahead of the MFMAs
+  constexpr int BK = 128;                      // reduction depth of one stage = one scale block = two MFMA steps
+  constexpr int NS = 2;                        // stages in the LDS ring
   constexpr int STAGE = (BM + BN) * BK;
-  constexpr int LA = BM / 16, LB = BN / 16;    // 1 KiB wave-loads (16 rows x 64 B) per operand stage
+  constexpr int LA = BM / 8, LB = BN / 8;      // 1 KiB wave-loads (8 rows x 128 B: full cache lines) per operand stage
   constexpr int SLA = BM / 64, SLB = BN / 64;  // 256 B wave-loads per scale vector
   constexpr int DPW = (LA + LB) / NW;          // data loads per wave per stage
-  static_assert(BM % 128 == 0 && BN % 128 == 0 && LA % NW == 0 && LB % NW == 0 && SLA + SLB == NW,
+  constexpr int SPW = (SLA + SLB) / NW;        // scale loads per wave per stage
+  static_assert(BM % 128 == 0 && BN % 128 == 0 && LA % NW == 0 && LB % NW == 0 && (SLA + SLB) % NW == 0 && SLA % SPW == 0,
                 "every wave must issue the same number of loads per stage");
-  constexpr int SC_RING = 4;
+  constexpr int SC_RING = NS;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [NS][STAGE] operand stages | [SC_RING][BM+BN] fp32 scales
   __shared__ int s_pref[MODE == GEMM_M_GROUPED ? kMaxGroupsGemm + 1 : 1];
 
@@ -180,7 +186,23 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   auto decode = [&](int t, Tile& T) {
     if (MODE == GEMM_DENSE) {
       T.g = 0;
-      T.a_row0 = (t % p.tiles_a) * BM; T.b_row0 = (t / p.tiles_a) * BN;
+      // The 32 CUs of an XCD work on 32 consecutive logical tiles at a time; laying those out as
+      // a 4 x 8 block of the output makes them share 4 a-tiles and 8 b-tiles in that XCD's L2
+      // instead of 32 a-tiles and 1 b-tile.
+      int ta, tb;
+      const int full_a = p.tiles_a & ~3, full_b = p.tiles_b & ~7;
+      const int nblk = (full_a >> 2) * (full_b >> 3);
+      if (t < nblk * 32) {
+        const int blk = t >> 5, in = t & 31;
+        ta = (blk % (full_a >> 2)) * 4 + (in & 3);
+        tb = (blk / (full_a >> 2)) * 8 + (in >> 2);
+      } else {  // ragged fringe: remaining columns of tiles, then remaining rows
+        const int r = t - nblk * 32;
+        const int fringe_b = p.tiles_b - full_b;  // extra b-tiles, all a-tiles
+        if (r < fringe_b * p.tiles_a) { ta = r % p.tiles_a; tb = full_b + r / p.tiles_a; }
+        else { const int r2 = r - fringe_b * p.tiles_a; ta = full_a + r2 % (p.tiles_a - full_a); tb = r2 / (p.tiles_a - full_a); }
+      }
+      T.a_row0 = ta * BM; T.b_row0 = tb * BN;
       T.a_lim = (int)p.rows_a; T.b_lim = (int)p.rows_b; T.k_begin = 0; T.k_len = (int)p.red; T.kb0 = 0;
     } else if (MODE == GEMM_M_GROUPED) {
       const int q = t / p.tiles_b;
@@ -209,19 +231,22 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   };
 
   // ---- LDS addressing ----
-  // A stage holds rows of 64 bytes (4 chunks of 16).  Row r keeps logical chunk c at position
-  // c ^ fs(r), fs(r) = ((r>>1)&3) ^ ((r>>3)&1), which spreads the ds_read_b128 of 8 or 16
-  // consecutive rows over all banks.  Direct-to-LDS wave-load q covers rows 16q..16q+15 (1 KiB):
-  // lane -> row 16q + lane/4, position lane%4; fs depends on row%16 = lane/4 only, so one per-lane
-  // offset serves every load and the rest of the address is uniform (scalar offset).
-  const int fs_ld = ((lane >> 3) & 3) ^ ((lane >> 5) & 1);
-  const int chunk = (lane & 3) ^ fs_ld;
-  const uint32_t va = (uint32_t)(lane >> 2) * (uint32_t)p.lda + chunk * 16;
-  const uint32_t vb = (uint32_t)(lane >> 2) * (uint32_t)p.ldb + chunk * 16;
-  const int fs_rd = (((lane & 31) >> 1) & 3) ^ (((lane & 31) >> 3) & 1);
-  const int roff = (lane & 31) * 64;
-  const int coff0 = roff + ((((lane >> 5) * 2 + 0) ^ fs_rd) << 4);
-  const int coff1 = roff + ((((lane >> 5) * 2 + 1) ^ fs_rd) << 4);
+  // A stage holds rows of 128 bytes (8 chunks of 16).  Row r keeps logical chunk c at position
+  // c ^ fs(r), fs(r) = (r&7) ^ ((r>>3)&1), which spreads the ds_read_b128 of 8 or 16 consecutive
+  // rows over all banks.  Direct-to-LDS wave-load q covers rows 8q..8q+7 (1 KiB, eight full
+  // 128-byte lines): lane -> row 8q + lane/8, position lane%8, i.e. logical chunk
+  // (lane%8) ^ (lane/8) ^ (q&1).  A wave's loads q = w, w+NW, ... all have the parity of w, so one
+  // per-lane offset serves them all and the rest of the address is uniform (scalar offset).
+  const int chunk = (lane & 7) ^ (lane >> 3) ^ (wave & 1);
+  const uint32_t va = (uint32_t)(lane >> 3) * (uint32_t)p.lda + chunk * 16;
+  const uint32_t vb = (uint32_t)(lane >> 3) * (uint32_t)p.ldb + chunk * 16;
+  const int fs_rd = (lane & 7) ^ ((lane >> 3) & 1);
+  const int roff = (lane & 31) * 128;
+  int coff[2][2];  // [MFMA step][half]: the lane's two chunks of a row for that step
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) coff[ks][h] = roff + (((ks * 4 + (lane >> 5) * 2 + h) ^ fs_rd) << 4);
 
   const v4i rs_a = make_rsrc(p.a, (uint32_t)p.a_bytes);
   const v4i rs_sa = make_rsrc(p.sa, (uint32_t)p.sa_bytes);
@@ -229,28 +254,30 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   const uint32_t pitch = (uint32_t)p.ldo * esz;
   const bool pair_ok = p.out_dtype != PT_F32 && (p.ldo & 1) == 0 && (((uintptr_t)p.out) & 3) == 0;
 
-  // ---- loader state: walks (tile, step) pairs NS-1 stages ahead of the MFMAs ----
+  // ---- loader: walks (tile, 128-block) pairs ahead of the MFMAs and keeps the LDS ring full ----
   Tile L;
   int lt = t_first - t_step, l_it = 0, l_nk = 0, n_issued = 0;
   v4i rs_b = rs_a, rs_sb = rs_sa;
-  uint32_t vs = 0;      // this wave's per-lane scale offset (bytes) at step 0 of the loader's tile
-  bool l_in_a = true;   // the scale vector this wave fetches: a (waves < SLA) or b
-  auto issue_stage = [&]() -> bool {
+  uint32_t vs[SPW];  // this wave's per-lane scale offsets (bytes) at step 0 of the loader's tile
+  auto issue_stage = [&]() {
     while (l_it >= l_nk) {
       lt += t_step;
-      if (lt >= t_end) return false;
+      if (lt >= t_end) return;
       decode(lt, L);
       l_it = 0;
-      l_nk = 2 * ((L.k_len + 127) >> 7);
+      l_nk = (L.k_len + 127) >> 7;
       rs_b = make_rsrc(p.b + (MODE == GEMM_M_GROUPED ? (int64_t)L.g * p.b_stride_g : 0), (uint32_t)p.b_bytes);
       rs_sb = make_rsrc(p.sb + (MODE == GEMM_M_GROUPED ? (int64_t)L.g * p.sb_stride_g : 0), (uint32_t)p.sb_bytes);
-      l_in_a = wave < SLA;
-      if (l_in_a) {
-        const int r = L.a_row0 + 64 * wave + lane;
-        vs = (uint32_t)(((int64_t)(r >> p.sa_shift) * p.sa_rs + (int64_t)L.kb0 * p.sa_ks) * 4);
-      } else {
-        const int r = L.b_row0 + 64 * (wave - SLA) + lane;
-        vs = (uint32_t)(((int64_t)(r >> p.sb_shift) * p.sb_rs + (int64_t)L.kb0 * p.sb_ks) * 4);
+#pragma unroll
+      for (int u = 0; u < SPW; ++u) {
+        const int q = wave * SPW + u;  // scale wave-load index: a for q < SLA, b after
+        if (q < SLA) {
+          const int r = L.a_row0 + 64 * q + lane;
+          vs[u] = (uint32_t)(((int64_t)(r >> p.sa_shift) * p.sa_rs + (int64_t)L.kb0 * p.sa_ks) * 4);
+        } else {
+          const int r = L.b_row0 + 64 * (q - SLA) + lane;
+          vs[u] = (uint32_t)(((int64_t)(r >> p.sb_shift) * p.sb_rs + (int64_t)L.kb0 * p.sb_ks) * 4);
+        }
       }
     }
     const int st = n_issued % NS;
@@ -258,36 +285,96 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
     const bool in = (int)(koff + chunk * 16) < L.k_len;  // false only in a ragged last 128-block
     const uint32_t sA = lds_base + st * STAGE, sB = sA + BM * BK;
     const int a_rows = L.a_lim - L.a_row0;  // rows past the end of a ragged group are not fetched
+    const uint32_t soA = (uint32_t)L.a_row0 * (uint32_t)p.lda + L.k_begin + koff;
+    const uint32_t soB = (uint32_t)L.b_row0 * (uint32_t)p.ldb + L.k_begin + koff;
 #pragma unroll
     for (int q0 = 0; q0 < LA; q0 += NW) {
       const int q = q0 + wave;
-      dma16(rs_a, (in && 16 * q < a_rows) ? va : kOob, (uint32_t)(L.a_row0 + 16 * q) * (uint32_t)p.lda + L.k_begin + koff,
-            sA + q * 1024);
+      dma16(rs_a, (in && 8 * q < a_rows) ? va : kOob, soA + (uint32_t)(8 * q) * (uint32_t)p.lda, sA + q * 1024);
     }
 #pragma unroll
     for (int q0 = 0; q0 < LB; q0 += NW) {
       const int q = q0 + wave;
-      dma16(rs_b, in ? vb : kOob, (uint32_t)(L.b_row0 + 16 * q) * (uint32_t)p.ldb + L.k_begin + koff, sB + q * 1024);
+      dma16(rs_b, in ? vb : kOob, soB + (uint32_t)(8 * q) * (uint32_t)p.ldb, sB + q * 1024);
     }
-    if ((l_it & 1) == 0) {
-      const uint32_t sc = sc_base + ((n_issued >> 1) % SC_RING) * (BM + BN) * 4 + wave * 256;
-      if (l_in_a) dma4(rs_sa, vs, (uint32_t)((l_it >> 1) * p.sa_ks * 4), sc);
-      else        dma4(rs_sb, vs, (uint32_t)((l_it >> 1) * p.sb_ks * 4), sc);
+    {
+      const uint32_t sc = sc_base + st * (BM + BN) * 4;
+#pragma unroll
+      for (int u = 0; u < SPW; ++u) {
+        const int q = wave * SPW + u;
+        if (q < SLA) dma4(rs_sa, vs[u], (uint32_t)(l_it * p.sa_ks * 4), sc + q * 256);
+        else         dma4(rs_sb, vs[u], (uint32_t)(l_it * p.sb_ks * 4), sc + q * 256);
+      }
     }
     ++l_it;
     ++n_issued;
-    return true;
+  };
+  // ---- L2 prefetcher: a third cursor, p.pf_dist 128-blocks ahead of the loader.  HBM latency is
+  // longer than the 1.5 stages of lookahead the LDS ring can hold, so the lines of a stage are
+  // pulled into L2 early by touching one dword of each 128-byte line (direct-to-LDS loads into a
+  // sink area: no VGPR is written behind the compiler's back).  Each wave touches the lines its
+  // own later stage loads will fetch: lane x -> load x/8 of the wave, row x%8. ----
+  Tile Pf;
+  int pt = t_first - t_step, p_it = 0, p_nk = 0;
+  v4i rs_b_pf = rs_a;
+  const uint32_t pf_sink = sc_base + NS * (BM + BN) * 4;
+  const bool pfa_ok = (lane >> 3) < LA / NW, pfb_ok = (lane >> 3) < LB / NW;
+  const uint32_t vpa = (uint32_t)(8 * (wave + NW * (lane >> 3)) + (lane & 7)) * (uint32_t)p.lda;
+  const uint32_t vpb = (uint32_t)(8 * (wave + NW * (lane >> 3)) + (lane & 7)) * (uint32_t)p.ldb;
+  auto prefetch_stage = [&]() {
+    while (p_it >= p_nk) {
+      pt += t_step;
+      if (pt >= t_end) return;
+      decode(pt, Pf);
+      p_it = 0;
+      p_nk = (Pf.k_len + 127) >> 7;
+      rs_b_pf = make_rsrc(p.b + (MODE == GEMM_M_GROUPED ? (int64_t)Pf.g * p.b_stride_g : 0), (uint32_t)p.b_bytes);
+    }
+    const uint32_t koff = (uint32_t)p_it * BK;
+    const int a_rows = Pf.a_lim - Pf.a_row0;
+    const bool a_in = pfa_ok && 8 * (wave + NW * (lane >> 3)) < a_rows;
+    dma4(rs_a, a_in ? vpa : kOob, (uint32_t)Pf.a_row0 * (uint32_t)p.lda + Pf.k_begin + koff, pf_sink);
+    dma4(rs_b_pf, pfb_ok ? vpb : kOob, (uint32_t)Pf.b_row0 * (uint32_t)p.ldb + Pf.k_begin + koff, pf_sink + 256);
+    ++p_it;
+  };
+
+  // Wait until stage `s` has landed for this wave.  Loads return in order, so it is enough that
+  // at most the operand and scale loads of the one stage issued after it are outstanding (its
+  // prefetch touches were issued before them and are older).  Stores of an earlier epilogue can
+  // only make the wait longer, never too short.
+  auto wait_stage = [&](int s) {
+    if (n_issued - s - 1 >= 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DPW + SPW) : "memory");
+    else wait_all_vmem();
+  };
+
+  auto read_frags = [&](int s, int ks, v8i* af, v8i* bf) {
+    const uint8_t* sA = lds + (s % NS) * STAGE + wm0 * BK;
+    const uint8_t* sB = lds + (s % NS) * STAGE + BM * BK + wn0 * BK;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const uint4 lo = *(const uint4*)(sA + i * 32 * BK + coff[ks][0]);
+      const uint4 hi = *(const uint4*)(sA + i * 32 * BK + coff[ks][1]);
+      af[i] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const uint4 lo = *(const uint4*)(sB + j * 32 * BK + coff[ks][0]);
+      const uint4 hi = *(const uint4*)(sB + j * 32 * BK + coff[ks][1]);
+      bf[j] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    }
   };
 
 #pragma unroll 1
-  for (int s = 0; s < NS - 1; ++s) issue_stage();
+  for (int s = 0; s < NS + p.pf_dist; ++s) prefetch_stage();
+#pragma unroll 1
+  for (int s = 0; s < NS; ++s) issue_stage();
 
-  int gs = 0;  // global step = index of the stage the MFMAs consume next
+  int gb = 0;  // global 128-block counter: the stage the MFMAs consume next
   Tile C;
 #pragma unroll 1
   for (int t = t_first; t < t_end; t += t_step) {
     decode(t, C);
-    const int nk = 2 * ((C.k_len + 127) >> 7);
+    const int nk = (C.k_len + 127) >> 7;
     // Waves whose whole row range lies past the end of a ragged group skip the MFMAs (they still
     // take part in the loads and barriers).
     const bool wave_active = C.a_row0 + wm0 < C.a_lim;
@@ -300,54 +387,44 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    int sca[TM], scb[TN];
 #pragma unroll 1
-    for (int it = 0; it < nk; ++it, ++gs) {
-      // Stage gs must have landed.  Loads return in order, so it is enough that at most the loads
-      // of the stages issued after it are outstanding: two stages = 2*DPW + 1 loads per wave (one
-      // of any two consecutive stages carries a scale load).  Stores of a previous epilogue may
-      // still be in flight and can only make this wait longer, never too short.
-      const int ahead = n_issued - gs - 1;
-      if (ahead >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DPW + 1) : "memory");
-      else if (ahead == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DPW) : "memory");
-      else wait_all_vmem();
-      __syncthreads();  // everybody's share has landed; everybody is done reading stage gs-1
-      issue_stage();    // refill the stage that was consumed in step gs-1
+    for (int it = 0; it < nk; ++it, ++gb) {
+      wait_stage(gb);
+      __syncthreads();  // everybody's share of stage gb has landed
+      v8i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+      int sca[TM], scb[TN];
       if (wave_active) {
-        if ((it & 1) == 0) {
-          const float* scA = sc_lds + ((gs >> 1) % SC_RING) * (BM + BN);
-          const float* scB = scA + BM;
+        const float* scA = sc_lds + (gb % NS) * (BM + BN);
+        const float* scB = scA + BM;
 #pragma unroll
-          for (int i = 0; i < TM; ++i) sca[i] = (int)(__float_as_uint(scA[wm0 + i * 32 + (lane & 31)]) >> 23);
+        for (int i = 0; i < TM; ++i) sca[i] = (int)(__float_as_uint(scA[wm0 + i * 32 + (lane & 31)]) >> 23);
 #pragma unroll
-          for (int j = 0; j < TN; ++j) scb[j] = (int)(__float_as_uint(scB[wn0 + j * 32 + (lane & 31)]) >> 23);
-        }
-        const uint8_t* sA = lds + (gs % NS) * STAGE + wm0 * BK;
-        const uint8_t* sB = lds + (gs % NS) * STAGE + BM * BK + wn0 * BK;
-        v8i af[TM], bf[TN];
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const uint4 lo = *(const uint4*)(sA + i * 32 * BK + coff0);
-          const uint4 hi = *(const uint4*)(sA + i * 32 * BK + coff1);
-          af[i] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-        }
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          const uint4 lo = *(const uint4*)(sB + j * 32 * BK + coff0);
-          const uint4 hi = *(const uint4*)(sB + j * 32 * BK + coff1);
-          bf[j] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-        }
+        for (int j = 0; j < TN; ++j) scb[j] = (int)(__float_as_uint(scB[wn0 + j * 32 + (lane & 31)]) >> 23);
+        read_frags(gb, 0, fa0, fb0);
+        read_frags(gb, 1, fa1, fb1);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf[j], acc[i][j], 0, 0, 0, sca[i], 0, scb[j]);
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa0[i], fb0[j], acc[i][j], 0, 0, 0, sca[i], 0, scb[j]);
+      }
+      // Every wave has pulled both steps' fragments of stage gb into registers: its ring slot can
+      // be refilled now, half a stage before the next barrier (the loads get 1.5 stages to land).
+      __syncthreads();
+      if (p.pf_dist > 0) prefetch_stage();
+      issue_stage();
+      if (wave_active) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa1[i], fb1[j], acc[i][j], 0, 0, 0, sca[i], 0, scb[j]);
       }
     }
 
     // ---- epilogue ----
     if (!wave_active) continue;
-    if (MODE == GEMM_K_GROUPED && nk == 0 && p.accumulate) continue;
+    if (MODE == GEMM_K_GROUPED && nk == 0 && ACC) continue;
     // The descriptor ends after the tile's last valid row: stores to ragged rows are dropped.
     char* outp = (char*)p.out + (MODE == GEMM_K_GROUPED ? (int64_t)C.g * p.out_stride_g * esz : 0);
     const __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(outp, 0, (int)((uint32_t)C.a_lim * pitch), kRsrcFlags);
@@ -359,21 +436,21 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
       for (int j = 0; j < TN; ++j) {
         const uint32_t voff = colw + j * 32 < C.b_lim ? (uint32_t)(4 * (lane >> 5) + odd) * pitch + (uint32_t)(((lane & 31) & ~1) + j * 32) * 2 : kOob;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) store_pairs_bf16(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, p.accumulate, odd);
+        for (int i = 0; i < TM; ++i) store_pairs_bf16(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC, odd);
       }
     } else if (p.out_dtype == PT_F32) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const uint32_t voff = colw + j * 32 < C.b_lim ? (uint32_t)(4 * (lane >> 5)) * pitch + (uint32_t)((lane & 31) + j * 32) * 4 : kOob;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) store_f32(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, p.accumulate);
+        for (int i = 0; i < TM; ++i) store_f32(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC);
       }
     } else {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const uint32_t voff = colw + j * 32 < C.b_lim ? (uint32_t)(4 * (lane >> 5)) * pitch + (uint32_t)((lane & 31) + j * 32) * 2 : kOob;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) store_single_bf16(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, p.accumulate);
+        for (int i = 0; i < TM; ++i) store_single_bf16(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC);
       }
     }
   }
@@ -382,13 +459,13 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
 
 static int g_num_cus = 0;
 
-template <int MODE, int BM, int BN, int WGM, int WGN>
+template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC>
 static int launch_one(GemmArgs a, hipStream_t stream) {
   constexpr int threads = WGM * WGN * 64;
-  constexpr size_t lds = (size_t)4 * (BM + BN) * 64 + 4 * (BM + BN) * 4;
+  constexpr size_t lds = (size_t)2 * (BM + BN) * 128 + 2 * (BM + BN) * 4 + 512;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)fp8_gemm_nt_persistent_kernel<MODE, BM, BN, WGM, WGN>,
+    hipError_t e = hipFuncSetAttribute((const void*)fp8_gemm_nt_persistent_kernel<MODE, BM, BN, WGM, WGN, ACC>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { set_error("gemm: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); return PT_ERR_LAUNCH; }
     attr_set = true;
@@ -399,6 +476,7 @@ static int launch_one(GemmArgs a, hipStream_t stream) {
       n = 256;
     g_num_cus = n;
   }
+  { const char* e = getenv("PT_GEMM_PF"); a.pf_dist = e ? atoi(e) : 0; if (a.pf_dist < 0) a.pf_dist = 0; }
   a.tiles_a = (int)cdiv(a.rows_a, BM);
   a.tiles_b = (int)cdiv(a.rows_b, BN);
   int64_t upper;
@@ -409,24 +487,26 @@ static int launch_one(GemmArgs a, hipStream_t stream) {
   PT_REQUIRE(upper < (1ll << 30), "gemm: too many tiles");
   int64_t blocks = (g_num_cus + 7) / 8 * 8;
   if (upper < blocks) blocks = (upper + 7) / 8 * 8;
-  hipLaunchKernelGGL((fp8_gemm_nt_persistent_kernel<MODE, BM, BN, WGM, WGN>), dim3((unsigned)blocks), dim3(threads), lds, stream, a);
+  hipLaunchKernelGGL((fp8_gemm_nt_persistent_kernel<MODE, BM, BN, WGM, WGN, ACC>), dim3((unsigned)blocks), dim3(threads), lds, stream, a);
   return check_launch("fp8_gemm_nt_persistent_kernel");
 }
 
 template <int BM, int BN, int WGM, int WGN>
 static int launch_mode(const GemmArgs& a, hipStream_t stream) {
   switch (a.mode) {
-    case GEMM_DENSE: return launch_one<GEMM_DENSE, BM, BN, WGM, WGN>(a, stream);
-    case GEMM_M_GROUPED: return launch_one<GEMM_M_GROUPED, BM, BN, WGM, WGN>(a, stream);
-    default: return launch_one<GEMM_K_GROUPED, BM, BN, WGM, WGN>(a, stream);
+    case GEMM_DENSE: return launch_one<GEMM_DENSE, BM, BN, WGM, WGN, false>(a, stream);
+    case GEMM_M_GROUPED: return launch_one<GEMM_M_GROUPED, BM, BN, WGM, WGN, false>(a, stream);
+    default:
+      return a.accumulate ? launch_one<GEMM_K_GROUPED, BM, BN, WGM, WGN, true>(a, stream)
+                          : launch_one<GEMM_K_GROUPED, BM, BN, WGM, WGN, false>(a, stream);
   }
 }
 
 int launch_gemm_persistent(const GemmArgs& a, int variant, hipStream_t stream) {
   PT_REQUIRE(a.mode != GEMM_M_GROUPED || a.G <= kMaxGroupsGemm, "gemm: at most %d groups", kMaxGroupsGemm);
   switch (variant) {
-    case 0: return launch_mode<256, 256, 2, 4>(a, stream);
-    case 1: return launch_mode<128, 128, 2, 2>(a, stream);
+    case 0: return launch_mode<256, 256, 2, 4>(a, stream);  // 8 waves, 128 x 64 per wave
+    case 1: return launch_mode<256, 256, 2, 2>(a, stream);  // 4 waves, 128 x 128 per wave
   }
   PT_REQUIRE(false, "gemm: unknown variant %d", variant);
 }
