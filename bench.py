@@ -27,6 +27,11 @@ if ROOT not in sys.path:
 FP8_DENSE_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
 HBM_PEAK_GBS = 8000.0
 
+# Average HBM bytes moved by one GEMM launch (fetch + write), from the FETCH_SIZE / WRITE_SIZE
+# counter runs summarised under profiles/ (scaled by the same counters' readings for a plain copy
+# of known size).  None for a workload that has no counter run.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-30b-a3b-moe": 855e6}
+
 WORKLOADS = {
     # name: (kind, hidden, intermediate, experts, top_k, tokens, zipf)
     "qwen3-30b-a3b-moe": ("fused", 2048, 768, 128, 8, 8192, None),
@@ -159,6 +164,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cached-weights", action="store_true",
                     help="also report a step time with the FP8 weight cache kept across steps")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="after the timed region launch gather_rows_kernel as a plain copy of 256 MiB "
+                         "(identity index) three times: the known-size kernel that FETCH_SIZE / "
+                         "WRITE_SIZE readings of a `rocprofv3 --pmc` run are scaled by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU's share of the expert path; run with --gpus 1 "
@@ -222,6 +231,17 @@ def main():
         torch.cuda.synchronize()
         extra["ms_per_step_weights_cached"] = (time.perf_counter() - t1) / args.steps * 1e3
 
+    if args.calibrate_copy:
+        cr, ch = 65536, 2048  # 65536 rows x 2048 bf16 = 256 MiB read + 256 MiB written (+ 512 KiB of indices)
+        csrc = torch.randn((cr, ch), device="cuda").bfloat16()
+        cdst = torch.empty_like(csrc)
+        cidx = torch.arange(cr, device="cuda", dtype=torch.int64)
+        for _ in range(3):
+            _lib.call("pt_gather_rows", csrc.data_ptr(), ch, cdst.data_ptr(), ch, cidx.data_ptr(), cr, ch, 2,
+                      _lib.stream_ptr())
+        torch.cuda.synchronize()
+        assert torch.equal(csrc, cdst)
+
     result = {
         "metric": "MoE-layer fwd+bwd TFLOP/s (FP8 grouped-expert path, Qwen3-30B-A3B shape, 1 GPU)"
         if args.workload == "qwen3-30b-a3b-moe" else f"MoE-layer fwd+bwd TFLOP/s ({args.workload})",
@@ -243,12 +263,14 @@ def main():
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "fp8_gemm_nt_kernel (all grouped GEMM launches of the step: fwd, dgrad, wgrad)",
+            "kernel": "fp8_gemm_nt_persistent_kernel (every GEMM launch of the step: fwd, dgrad, wgrad)",
             "achieved": achieved,
             "peak": FP8_DENSE_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / FP8_DENSE_PEAK_TFLOPS,
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
+            "algorithmic_flop_per_launch": flops / max(gemm_launches / max(args.steps, 1), 1),
+            "avg_launch_ms": gemm_ms / max(gemm_launches, 1),
             "launches_per_step": gemm_launches / max(args.steps, 1),
             "gemm_ms_per_step": gemm_ms / max(args.steps, 1),
             "per_entry_point_ms_per_step": {k2: v["ms_total"] / args.steps for k2, v in gs.items()},
