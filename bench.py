@@ -200,8 +200,10 @@ def main():
             p.grad = None
         tok = tokens.detach().requires_grad_(True)
         out = forward_stage3(mod, tok, eidx, E)
-        out.backward(dyc)
-        return tok.grad
+        # weight gradients are written to .grad by the wgrad GEMM itself; the token gradient is
+        # taken directly (a leaf's .grad would cost a clone that no training step performs)
+        (dtok,) = torch.autograd.grad(out, tok, dyc)
+        return dtok
 
     for _ in range(args.warmup):
         step()

@@ -195,6 +195,16 @@ int pt_silu_mul_fwd(const void* gate, const void* up, void* out, int64_t n, int 
 /* _silu_mul_bwd_kernel, silu_mul.py:52-87 */
 int pt_silu_mul_bwd(const void* grad_out, const void* gate, const void* up, void* grad_gate,
                     void* grad_up, int64_t n, int dtype, pt_stream_t stream);
+/* The same two kernels on [rows, cols] views with their own leading dimensions (in elements), so
+ * that the halves of a fused gate_up buffer are read in place and both gradients land in one
+ * [rows, 2*cols] buffer: replaces the .contiguous() copies around silu_mul in
+ * Qwen35MoeExperts.forward (models/qwen35_moe.py:196-199) and their autograd backward. */
+int pt_silu_mul_fwd_2d(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, void* out,
+                       int64_t ld_out, int64_t rows, int64_t cols, int dtype, pt_stream_t stream);
+int pt_silu_mul_bwd_2d(const void* grad_out, int64_t ld_grad_out, const void* gate, int64_t ld_gate,
+                       const void* up, int64_t ld_up, void* grad_gate, int64_t ld_grad_gate,
+                       void* grad_up, int64_t ld_grad_up, int64_t rows, int64_t cols, int dtype,
+                       pt_stream_t stream);
 /* gate_up[M,2N] interleaved -> out[M,N]; n = M*N.  _clamped_swiglu_fwd_kernel,
  * clamped_swiglu.py:18-46 */
 int pt_clamped_swiglu_fwd(const void* gate_up, void* out, int64_t n, float alpha, float limit,

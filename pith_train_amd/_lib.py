@@ -46,6 +46,8 @@ SIGNATURES = {
     "pt_adjust_expand_idx": (c_int, [P, P, P, I64, P, I32, I64, P]),
     "pt_silu_mul_fwd": (c_int, [P, P, P, I64, c_int, P]),
     "pt_silu_mul_bwd": (c_int, [P, P, P, P, P, I64, c_int, P]),
+    "pt_silu_mul_fwd_2d": (c_int, [P, I64, P, I64, P, I64, I64, I64, c_int, P]),
+    "pt_silu_mul_bwd_2d": (c_int, [P, I64, P, I64, P, I64, P, I64, P, I64, I64, I64, c_int, P]),
     "pt_clamped_swiglu_fwd": (c_int, [P, P, I64, F, F, c_int, P]),
     "pt_clamped_swiglu_bwd": (c_int, [P, P, P, I64, F, F, c_int, P]),
     "pt_indexed_bias_add_fwd": (c_int, [P, P, P, P, I64, I64, c_int, P]),

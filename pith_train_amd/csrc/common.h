@@ -42,8 +42,13 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
 }
+// The conversion is an opaque instruction on purpose: written as a cast, the compiler folds a
+// preceding fp32 multiply into v_fma_mixlo_f16 (one rounding instead of fp32-then-fp16), which
+// makes the result depend on how each kernel happens to be scheduled.
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
-  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+  uint32_t r;
+  asm("v_cvt_f16_f32_e32 %0, %1" : "=v"(r) : "v"(f));
+  return r & 0xFFFFu;
 }
 
 // ---- storage types: 8-wide vector and scalar load/store with fp32 math ---------------------------

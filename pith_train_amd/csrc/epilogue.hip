@@ -8,10 +8,21 @@
 namespace pt {
 
 __device__ __forceinline__ float sigmoidf_fast(float x) {
-  return __builtin_amdgcn_rcpf(1.0f + __expf(-x));
+  return __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-x)));
 }
 
 // ---- silu_mul ---------------------------------------------------------------------------------
+// The arithmetic is spelled with explicit round-to-nearest operations so that every kernel that
+// uses it (flat and row-strided) produces the same bits whatever the compiler would contract.
+__device__ __forceinline__ float silu_mul_f(float g, float u) {
+  return __fmul_rn(__fmul_rn(g, sigmoidf_fast(g)), u);
+}
+__device__ __forceinline__ void silu_mul_b(float d, float g, float u, float& dg, float& du) {
+  const float sig = sigmoidf_fast(g);
+  const float silu = __fmul_rn(g, sig);
+  du = __fmul_rn(d, silu);
+  dg = __fmul_rn(__fmul_rn(__fmul_rn(d, u), sig), __fsub_rn(__fadd_rn(1.0f, g), silu));
+}
 template <typename S>
 __global__ __launch_bounds__(256) void silu_mul_fwd_kernel(const char* gate, const char* up, char* out, int64_t n) {
   const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
@@ -21,12 +32,12 @@ __global__ __launch_bounds__(256) void silu_mul_fwd_kernel(const char* gate, con
     S::load8(gate + i0 * S::kBytes, g);
     S::load8(up + i0 * S::kBytes, u);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) o[j] = g[j] * sigmoidf_fast(g[j]) * u[j];
+    for (int j = 0; j < 8; ++j) o[j] = silu_mul_f(g[j], u[j]);
     S::store8(out + i0 * S::kBytes, o);
   } else {
     for (int64_t i = i0; i < n; ++i) {
       const float g = S::load1(gate + i * S::kBytes), u = S::load1(up + i * S::kBytes);
-      S::store1(out + i * S::kBytes, g * sigmoidf_fast(g) * u);
+      S::store1(out + i * S::kBytes, silu_mul_f(g, u));
     }
   }
 }
@@ -36,12 +47,7 @@ __global__ __launch_bounds__(256) void silu_mul_bwd_kernel(const char* go, const
                                                            char* dgate, char* dup, int64_t n) {
   const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
   if (i0 >= n) return;
-  auto one = [](float d, float g, float u, float& dg, float& du) {
-    const float sig = sigmoidf_fast(g);
-    const float silu = g * sig;
-    du = d * silu;
-    dg = d * u * sig * (1.0f + g - silu);
-  };
+  auto one = [](float d, float g, float u, float& dg, float& du) { silu_mul_b(d, g, u, dg, du); };
   if (i0 + 8 <= n) {
     float d[8], g[8], u[8], dg[8], du[8];
     S::load8(go + i0 * S::kBytes, d);
@@ -57,6 +63,70 @@ __global__ __launch_bounds__(256) void silu_mul_bwd_kernel(const char* go, const
       one(S::load1(go + i * S::kBytes), S::load1(gate + i * S::kBytes), S::load1(up + i * S::kBytes), dg, du);
       S::store1(dgate + i * S::kBytes, dg);
       S::store1(dup + i * S::kBytes, du);
+    }
+  }
+}
+
+// ---- silu_mul on row-strided operands ---------------------------------------------------------------
+// gate / up / out (and their gradients) are [rows, cols] views with their own leading dimensions
+// (in elements), e.g. the two halves of a fused gate_up buffer.  One thread per 8-element chunk.
+struct Silu2dArgs {
+  const char *go, *gate, *up;
+  char *out, *dgate, *dup;
+  int64_t ld_go, ld_gate, ld_up, ld_out, ld_dgate, ld_dup;  // bytes
+  uint32_t rows, cols, chunks_per_row, total_chunks;
+  int vec;
+};
+
+template <typename S, bool BWD>
+__global__ __launch_bounds__(256) void silu_mul_2d_kernel(Silu2dArgs p) {
+  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+  if (c >= p.total_chunks) return;
+  const uint32_t r = c / p.chunks_per_row;
+  const uint32_t col = (c - r * p.chunks_per_row) * 8u;
+  const int64_t cb = (int64_t)col * S::kBytes;
+  const char* gp = p.gate + r * p.ld_gate + cb;
+  const char* upp = p.up + r * p.ld_up + cb;
+  float g[8], u[8];
+  const int nval = (p.cols - col) < 8u ? (int)(p.cols - col) : 8;
+  if (p.vec) {
+    S::load8(gp, g);
+    S::load8(upp, u);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      g[j] = j < nval ? S::load1(gp + j * S::kBytes) : 0.f;
+      u[j] = j < nval ? S::load1(upp + j * S::kBytes) : 0.f;
+    }
+  }
+  if (!BWD) {
+    float o[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = silu_mul_f(g[j], u[j]);
+    char* op = p.out + r * p.ld_out + cb;
+    if (p.vec) S::store8(op, o);
+    else
+      for (int j = 0; j < nval; ++j) S::store1(op + j * S::kBytes, o[j]);
+  } else {
+    float d[8], dg[8], du[8];
+    const char* dp = p.go + r * p.ld_go + cb;
+    if (p.vec) S::load8(dp, d);
+    else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) d[j] = j < nval ? S::load1(dp + j * S::kBytes) : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) silu_mul_b(d[j], g[j], u[j], dg[j], du[j]);
+    char* dgp = p.dgate + r * p.ld_dgate + cb;
+    char* dup = p.dup + r * p.ld_dup + cb;
+    if (p.vec) {
+      S::store8(dgp, dg);
+      S::store8(dup, du);
+    } else {
+      for (int j = 0; j < nval; ++j) {
+        S::store1(dgp + j * S::kBytes, dg[j]);
+        S::store1(dup + j * S::kBytes, du[j]);
+      }
     }
   }
 }
@@ -228,6 +298,62 @@ extern "C" int pt_silu_mul_bwd(const void* go, const void* gate, const void* up,
   PT_DISPATCH_ST(dtype, silu_mul_bwd_kernel,
                  <<<blocks8(n), 256, 0, s>>>((const char*)go, (const char*)gate, (const char*)up, (char*)dgate, (char*)dup, n));
   return check_launch("silu_mul_bwd");
+}
+
+static int silu_2d_setup(Silu2dArgs& a, int64_t rows, int64_t cols, int dtype, const char* what) {
+  PT_REQUIRE(rows > 0 && cols > 0, "%s: bad shape", what);
+  const int64_t cpr = cdiv(cols, 8);
+  PT_REQUIRE(rows * cpr < (1ll << 31), "%s: too many elements", what);
+  a.rows = (uint32_t)rows; a.cols = (uint32_t)cols; a.chunks_per_row = (uint32_t)cpr;
+  a.total_chunks = (uint32_t)(rows * cpr);
+  (void)dtype;
+  return PT_OK;
+}
+
+extern "C" int pt_silu_mul_fwd_2d(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, void* out,
+                                  int64_t ld_out, int64_t rows, int64_t cols, int dtype, pt_stream_t stream) {
+  if (rows == 0 || cols == 0) return PT_OK;
+  PT_REQUIRE(gate && up && out && ld_gate >= cols && ld_up >= cols && ld_out >= cols, "silu_mul_fwd_2d: bad arguments");
+  const int eb = dtype == PT_F32 ? 4 : 2;
+  Silu2dArgs a{};
+  if (int rc = silu_2d_setup(a, rows, cols, dtype, "silu_mul_fwd_2d")) return rc;
+  a.gate = (const char*)gate; a.up = (const char*)up; a.out = (char*)out;
+  a.ld_gate = ld_gate * eb; a.ld_up = ld_up * eb; a.ld_out = ld_out * eb;
+  a.vec = cols % 8 == 0 && aligned16(gate) && aligned16(up) && aligned16(out) && a.ld_gate % 16 == 0 &&
+          a.ld_up % 16 == 0 && a.ld_out % 16 == 0;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned blocks = (unsigned)cdiv((int64_t)a.total_chunks, 256);
+  switch (dtype) {
+    case PT_BF16: silu_mul_2d_kernel<st_bf16, false><<<blocks, 256, 0, s>>>(a); break;
+    case PT_F16:  silu_mul_2d_kernel<st_f16, false><<<blocks, 256, 0, s>>>(a); break;
+    case PT_F32:  silu_mul_2d_kernel<st_f32, false><<<blocks, 256, 0, s>>>(a); break;
+    default: PT_REQUIRE(false, "silu_mul_fwd_2d: unsupported dtype %d", dtype);
+  }
+  return check_launch("silu_mul_fwd_2d");
+}
+
+extern "C" int pt_silu_mul_bwd_2d(const void* go, int64_t ld_go, const void* gate, int64_t ld_gate, const void* up,
+                                  int64_t ld_up, void* dgate, int64_t ld_dgate, void* dup, int64_t ld_dup, int64_t rows,
+                                  int64_t cols, int dtype, pt_stream_t stream) {
+  if (rows == 0 || cols == 0) return PT_OK;
+  PT_REQUIRE(go && gate && up && dgate && dup && ld_go >= cols && ld_gate >= cols && ld_up >= cols && ld_dgate >= cols &&
+                 ld_dup >= cols, "silu_mul_bwd_2d: bad arguments");
+  const int eb = dtype == PT_F32 ? 4 : 2;
+  Silu2dArgs a{};
+  if (int rc = silu_2d_setup(a, rows, cols, dtype, "silu_mul_bwd_2d")) return rc;
+  a.go = (const char*)go; a.gate = (const char*)gate; a.up = (const char*)up; a.dgate = (char*)dgate; a.dup = (char*)dup;
+  a.ld_go = ld_go * eb; a.ld_gate = ld_gate * eb; a.ld_up = ld_up * eb; a.ld_dgate = ld_dgate * eb; a.ld_dup = ld_dup * eb;
+  a.vec = cols % 8 == 0 && aligned16(go) && aligned16(gate) && aligned16(up) && aligned16(dgate) && aligned16(dup) &&
+          a.ld_go % 16 == 0 && a.ld_gate % 16 == 0 && a.ld_up % 16 == 0 && a.ld_dgate % 16 == 0 && a.ld_dup % 16 == 0;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned blocks = (unsigned)cdiv((int64_t)a.total_chunks, 256);
+  switch (dtype) {
+    case PT_BF16: silu_mul_2d_kernel<st_bf16, true><<<blocks, 256, 0, s>>>(a); break;
+    case PT_F16:  silu_mul_2d_kernel<st_f16, true><<<blocks, 256, 0, s>>>(a); break;
+    case PT_F32:  silu_mul_2d_kernel<st_f32, true><<<blocks, 256, 0, s>>>(a); break;
+    default: PT_REQUIRE(false, "silu_mul_bwd_2d: unsupported dtype %d", dtype);
+  }
+  return check_launch("silu_mul_bwd_2d");
 }
 
 extern "C" int pt_clamped_swiglu_fwd(const void* gate_up, void* out, int64_t n, float alpha, float limit, int dtype,

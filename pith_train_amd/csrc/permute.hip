@@ -57,29 +57,55 @@ __global__ __launch_bounds__(256) void gr_hist_kernel(const int64_t* keys, int64
     for (int g = lane; g < G; g += 64) counts[w * G + g] = h[g];
 }
 
-// one workgroup: counts[W][G] -> exclusive bases in place; padded sizes, inclusive offsets, starts
-__global__ __launch_bounds__(1024) void gr_scan_kernel(int32_t* counts, int64_t W, int G, int alignment, int32_t* offs,
-                                                       int32_t* ks, int32_t* group_start /*[G]*/) {
-  __shared__ int32_t s_tot[kMaxGroups];
-  for (int g = threadIdx.x; g < G; g += blockDim.x) {
-    int32_t run = 0;
-    for (int64_t w = 0; w < W; ++w) {
-      const int32_t c = counts[w * G + g];
-      counts[w * G + g] = run;
-      run += c;
+// counts[W][G] -> exclusive bases over the chunks in place, one wavefront per group (64 chunks per
+// step, ranked with a wave prefix sum); the group's total goes to totals[g].
+__global__ __launch_bounds__(256) void gr_scan_chunks_kernel(int32_t* counts, int64_t W, int G, int32_t* totals) {
+  const int lane = threadIdx.x & 63;
+  const int g = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (g >= G) return;
+  int32_t run = 0;
+  for (int64_t w0 = 0; w0 < W; w0 += 64) {
+    const int64_t w = w0 + lane;
+    const int32_t c = w < W ? counts[w * G + g] : 0;
+    int32_t incl = c;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int32_t up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
     }
-    s_tot[g] = run;
+    if (w < W) counts[w * G + g] = run + incl - c;
+    run += __shfl(incl, 63);
   }
+  if (lane == 0) totals[g] = run;
+}
+
+// one workgroup: per-group totals (read from group_start) -> padded sizes, inclusive offsets, starts
+__global__ __launch_bounds__(1024) void gr_scan_groups_kernel(int G, int alignment, int32_t* offs, int32_t* ks,
+                                                              int32_t* group_start /*[G]: totals in, starts out*/) {
+  __shared__ int32_t s_part[1024];
+  const int t = threadIdx.x;
+  // thread t owns groups 2t and 2t+1 (G <= 2048)
+  int32_t p0 = 0, p1 = 0;
+  if (2 * t < G) p0 = (int32_t)(((int64_t)group_start[2 * t] + alignment - 1) / alignment * alignment);
+  if (2 * t + 1 < G) p1 = (int32_t)(((int64_t)group_start[2 * t + 1] + alignment - 1) / alignment * alignment);
+  s_part[t] = p0 + p1;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int64_t run = 0;
-    for (int g = 0; g < G; ++g) {
-      const int64_t padded = ((int64_t)s_tot[g] + alignment - 1) / alignment * alignment;
-      group_start[g] = (int32_t)run;
-      run += padded;
-      offs[g] = (int32_t)run;
-      ks[g] = (int32_t)padded;
-    }
+  for (int d = 1; d < 1024; d <<= 1) {
+    const int32_t add = t >= d ? s_part[t - d] : 0;
+    __syncthreads();
+    s_part[t] += add;
+    __syncthreads();
+  }
+  const int32_t excl = s_part[t] - (p0 + p1);
+  if (2 * t < G) {
+    group_start[2 * t] = excl;
+    offs[2 * t] = excl + p0;
+    ks[2 * t] = p0;
+  }
+  if (2 * t + 1 < G) {
+    group_start[2 * t + 1] = excl + p0;
+    offs[2 * t + 1] = excl + p0 + p1;
+    ks[2 * t + 1] = p1;
   }
 }
 
@@ -546,7 +572,8 @@ extern "C" int pt_group_rows(const int64_t* keys, int64_t m, int32_t G, int32_t 
   const size_t lds = (size_t)4 * G * sizeof(int32_t);
   fill_i32_kernel<<<(unsigned)cdiv(cap, 256), 256, 0, s>>>(src_of, cap, -1);
   gr_hist_kernel<<<blocks, 256, lds, s>>>(keys, m, G, counts);
-  gr_scan_kernel<<<1, 1024, 0, s>>>(counts, W, G, alignment, offs, ks, group_start);
+  gr_scan_chunks_kernel<<<(unsigned)cdiv(G, 4), 256, 0, s>>>(counts, W, G, group_start);
+  gr_scan_groups_kernel<<<1, 1024, 0, s>>>(G, alignment, offs, ks, group_start);
   gr_rank_kernel<<<blocks, 256, lds, s>>>(keys, m, G, bits_for(G), counts, group_start, reverse, src_of, cap);
   return check_launch("group_rows");
 }

@@ -24,7 +24,7 @@ from ..operators.clamped_swiglu import clamped_swiglu
 from ..operators.deepgemm_quantize import fp8cast_blockwise_transpose_batched
 from ..operators.grouped_linear import FP8GroupedLinearFunc, GroupedLinearFunc
 from ..operators.indexed_bias_add import indexed_bias_add
-from ..operators.silu_mul import silu_mul
+from ..operators.silu_mul import silu_mul, silu_mul_halves
 from ..operators.token_scatter import (
     group_indices,
     padded_index_gather,
@@ -79,9 +79,8 @@ class Qwen35MoeExperts(nn.Module):
         gi = precompute_group_indices(grouped_mm_offs, x.shape[0])
         kwargs = dict(grouped_mm_offs=grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, group_indices=gi)
         gate_up = self.gate_up_proj(x, **kwargs)
-        gate = gate_up[:, : self.moe_intermediate_size].contiguous()
-        up = gate_up[:, self.moe_intermediate_size :].contiguous()
-        return self.down_proj(silu_mul(gate, up), **kwargs)
+        # the halves are read in place (same arithmetic as silu_mul on contiguous copies)
+        return self.down_proj(silu_mul_halves(gate_up), **kwargs)
 
 
 class GptOssExperts(nn.Module):

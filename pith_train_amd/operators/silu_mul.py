@@ -50,3 +50,52 @@ class _SiLUMul(torch.autograd.Function):
 def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """Element-wise ``silu(gate) * up`` in the dtype of the inputs."""
     return _SiLUMul.apply(gate, up)
+
+
+class _SiLUMulHalves(torch.autograd.Function):
+    """``silu(gate_up[:, :I]) * gate_up[:, I:]`` without materialising the halves.
+
+    Same arithmetic as ``_SiLUMul``; the two halves are read in place through their row stride
+    and the backward writes both gradients into one ``[M, 2I]`` buffer, which removes the two
+    ``.contiguous()`` copies of ``Qwen35MoeExperts.forward`` (models/qwen35_moe.py:196-199) and
+    the zero-fill + slice-copy + add that autograd runs for them in backward.
+    """
+
+    @staticmethod
+    def forward(ctx, gate_up: torch.Tensor) -> torch.Tensor:
+        assert gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, f"bad gate_up shape {tuple(gate_up.shape)}"
+        assert gate_up.is_contiguous(), "gate_up must be contiguous"
+        _lib.require_cuda(gate_up)
+        rows, two_i = gate_up.shape
+        inter = two_i // 2
+        eb = gate_up.element_size()
+        ctx.save_for_backward(gate_up)
+        out = torch.empty((rows, inter), dtype=gate_up.dtype, device=gate_up.device)
+        _lib.call(
+            "pt_silu_mul_fwd_2d", gate_up.data_ptr(), two_i, gate_up.data_ptr() + inter * eb, two_i,
+            out.data_ptr(), inter, rows, inter, _lib.dtype_code(gate_up.dtype), _lib.stream_ptr(gate_up.device),
+        )  # fmt: skip
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        (gate_up,) = ctx.saved_tensors
+        rows, two_i = gate_up.shape
+        inter = two_i // 2
+        eb = gate_up.element_size()
+        assert grad_output.shape == (rows, inter), f"grad_output shape {tuple(grad_output.shape)}"
+        assert grad_output.dtype == gate_up.dtype, f"grad_output dtype {grad_output.dtype} != {gate_up.dtype}"
+        assert grad_output.is_contiguous(), "grad_output must be contiguous"
+        grad = torch.empty_like(gate_up)
+        _lib.call(
+            "pt_silu_mul_bwd_2d", grad_output.data_ptr(), inter, gate_up.data_ptr(), two_i,
+            gate_up.data_ptr() + inter * eb, two_i, grad.data_ptr(), two_i, grad.data_ptr() + inter * eb, two_i,
+            rows, inter, _lib.dtype_code(gate_up.dtype), _lib.stream_ptr(gate_up.device),
+        )  # fmt: skip
+        return grad
+
+
+def silu_mul_halves(gate_up: torch.Tensor) -> torch.Tensor:
+    """``silu_mul(gate_up[:, :I], gate_up[:, I:])`` for a fused ``[M, 2I]`` projection output
+    (concatenated halves), bit-identical to the two-tensor form."""
+    return _SiLUMulHalves.apply(gate_up)

@@ -51,6 +51,27 @@ def test_silu_mul(shape, dtype):
     assert torch.allclose(b.grad.float().cpu(), u32.grad, atol=1e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("rows,inter", [(8192, 768), (1000, 100), (3, 4), (129, 1408), (7, 5)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_silu_mul_halves_matches_two_tensor_form(rows, inter, dtype):
+    """The in-place-halves form is bit-identical (outputs and both gradients) to silu_mul on
+    contiguous copies of the halves, and within an ulp of the oracle."""
+    from pith_train_amd.operators.silu_mul import silu_mul, silu_mul_halves
+
+    g = torch.Generator().manual_seed(rows + inter)
+    gu = (torch.randn((rows, 2 * inter), generator=g) * 2).to(dtype)
+    do = torch.randn((rows, inter), generator=g).to(dtype)
+    a = gu.cuda().requires_grad_(True)
+    out = silu_mul_halves(a)
+    out.backward(do.cuda())
+    b = gu.cuda().requires_grad_(True)
+    ref = silu_mul(b[:, :inter].contiguous(), b[:, inter:].contiguous())
+    ref.backward(do.cuda())
+    assert torch.equal(out, ref)
+    assert torch.equal(a.grad, b.grad)
+    _close_ulp(out, E.silu_mul_fwd(gu[:, :inter].contiguous(), gu[:, inter:].contiguous()), dtype, "fwd")
+
+
 def test_silu_mul_asserts():
     from pith_train_amd.operators.silu_mul import silu_mul
 

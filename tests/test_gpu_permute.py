@@ -21,7 +21,8 @@ def _ts():
 
 SCATTER = [(1024, 8, 256, torch.bfloat16), (100, 4, 100, torch.float32), (5000, 128, 64, torch.bfloat16),
            (1, 8, 1, torch.float32), (777, 1, 128, torch.bfloat16), (4096, 64, 2048, torch.bfloat16),
-           (300, 300, 16, torch.float16), (65536, 128, 128, torch.bfloat16)]
+           (300, 300, 16, torch.float16), (65536, 128, 128, torch.bfloat16),
+           (40000, 2048, 8, torch.bfloat16), (20000, 1001, 8, torch.float32)]
 
 
 @pytest.mark.parametrize("m,G,H,dtype", SCATTER)
