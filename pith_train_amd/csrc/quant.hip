@@ -56,6 +56,46 @@ template <> struct Loader<float> {
   }
 };
 
+// The thread's 8x8 sub-block.  bf16 sources stay packed (two values per register, unpacked at
+// each use): half the registers of an fp32 copy, which is what lets enough wavefronts be
+// resident to keep HBM busy.
+template <typename T> struct Frag;
+template <> struct Frag<bf16_tag> {
+  uint32_t w[8][4];
+  __device__ __forceinline__ void load_row(int i, const void* p) {
+    const uint4 u = *reinterpret_cast<const uint4*>(p);
+    w[i][0] = u.x; w[i][1] = u.y; w[i][2] = u.z; w[i][3] = u.w;
+  }
+  __device__ __forceinline__ void zero_row(int i) { w[i][0] = w[i][1] = w[i][2] = w[i][3] = 0u; }
+  __device__ __forceinline__ void set(int i, int j, const void* p) {
+    const uint32_t b = *reinterpret_cast<const uint16_t*>(p);
+    w[i][j >> 1] = (j & 1) ? ((w[i][j >> 1] & 0x0000FFFFu) | (b << 16)) : ((w[i][j >> 1] & 0xFFFF0000u) | b);
+  }
+  __device__ __forceinline__ float get(int i, int j) const { return (j & 1) ? bf16_hi(w[i][j >> 1]) : bf16_lo(w[i][j >> 1]); }
+  // Compiler fence on the packed registers: values unpacked before it cannot be kept live
+  // across it, so each phase of the kernel unpacks again instead of holding 64 floats.
+  __device__ __forceinline__ void fence() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) fence_row(i);
+  }
+  __device__ __forceinline__ void fence_row(int i) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) asm volatile("" : "+v"(w[i][k]));
+  }
+};
+template <> struct Frag<float> {
+  float v[8][8];
+  __device__ __forceinline__ void load_row(int i, const void* p) { Loader<float>::load8(p, v[i]); }
+  __device__ __forceinline__ void zero_row(int i) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[i][j] = 0.f;
+  }
+  __device__ __forceinline__ void set(int i, int j, const void* p) { v[i][j] = *reinterpret_cast<const float*>(p); }
+  __device__ __forceinline__ float get(int i, int j) const { return v[i][j]; }
+  __device__ __forceinline__ void fence() {}
+  __device__ __forceinline__ void fence_row(int) {}
+};
+
 template <typename T, int AM, int BMODE, int BL, int BS>
 __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   __shared__ float s_colmax[4][128];
@@ -73,35 +113,31 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   const int64_t col0 = (int64_t)tc * 128 + cc * 8;
   const char* xb = reinterpret_cast<const char*>(p.x) + g * p.x_stride_g * Loader<T>::kBytes;
 
-  float v[8][8];
+  Frag<T> f;
   if (p.vec_in) {
     const bool col_ok = col0 < p.N;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      if (col_ok && row0 + i < p.M) {
-        Loader<T>::load8(xb + ((row0 + i) * p.ldx + col0) * Loader<T>::kBytes, v[i]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[i][j] = 0.f;
-      }
+      if (col_ok && row0 + i < p.M) f.load_row(i, xb + ((row0 + i) * p.ldx + col0) * Loader<T>::kBytes);
+      else f.zero_row(i);
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 8; ++i) {
+      f.zero_row(i);
 #pragma unroll
       for (int j = 0; j < 8; ++j)
-        v[i][j] = (row0 + i < p.M && col0 + j < p.N)
-                      ? Loader<T>::load1(xb + ((row0 + i) * p.ldx + col0 + j) * Loader<T>::kBytes)
-                      : 0.f;
+        if (row0 + i < p.M && col0 + j < p.N) f.set(i, j, xb + ((row0 + i) * p.ldx + col0 + j) * Loader<T>::kBytes);
+    }
   }
 
   // ---- reductions ------------------------------------------------------------------------
   float rowmax[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    float m = fabsf(v[i][0]);
+    float m = fabsf(f.get(i, 0));
 #pragma unroll
-    for (int j = 1; j < 8; ++j) m = fmaxf(m, fabsf(v[i][j]));
+    for (int j = 1; j < 8; ++j) m = fmaxf(m, fabsf(f.get(i, j)));
     rowmax[i] = m;
   }
   if (AM == A_ROW) {
@@ -109,13 +145,14 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
     for (int i = 0; i < 8; ++i) rowmax[i] = row16_allmax(rowmax[i]);
   }
 
+  f.fence();
   float colmax[8];
   if (BMODE == B_COL) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      float m = fabsf(v[0][j]);
+      float m = fabsf(f.get(0, j));
 #pragma unroll
-      for (int i = 1; i < 8; ++i) m = fmaxf(m, fabsf(v[i][j]));
+      for (int i = 1; i < 8; ++i) m = fmaxf(m, fabsf(f.get(i, j)));
       m = fmaxf(m, __shfl_xor(m, 16));
       m = fmaxf(m, __shfl_xor(m, 32));
       colmax[j] = m;
@@ -149,11 +186,13 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   }
 
   // ---- same-orientation output -----------------------------------------------------------
+  f.fence();
   {
     uint8_t* ab = p.a_out + g * p.a_stride_g;
     const int64_t nb = p.tiles_n;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
+      f.fence_row(i);
       float rcp;
       if (AM == A_ROW) {
         const float s = fp8_scale_from_amax(rowmax[i], rcp);
@@ -161,8 +200,8 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
       } else {
         rcp = blk_rcp;
       }
-      const uint32_t lo = cvt4_e4m3(v[i][0] * rcp, v[i][1] * rcp, v[i][2] * rcp, v[i][3] * rcp);
-      const uint32_t hi = cvt4_e4m3(v[i][4] * rcp, v[i][5] * rcp, v[i][6] * rcp, v[i][7] * rcp);
+      const uint32_t lo = cvt4_e4m3(f.get(i, 0) * rcp, f.get(i, 1) * rcp, f.get(i, 2) * rcp, f.get(i, 3) * rcp);
+      const uint32_t hi = cvt4_e4m3(f.get(i, 4) * rcp, f.get(i, 5) * rcp, f.get(i, 6) * rcp, f.get(i, 7) * rcp);
       if (row0 + i < p.M) {
         uint8_t* dst = ab + (row0 + i) * p.N + col0;
         if (p.vec_out) {
@@ -179,6 +218,7 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   }
 
   // ---- twin ---------------------------------------------------------------------------------
+  f.fence();
   float crcp[8];
   if (BMODE == B_COL) {
 #pragma unroll
@@ -199,8 +239,9 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
     uint8_t* bb = p.b_out + g * p.b_stride_g;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const uint32_t lo = cvt4_e4m3(v[i][0] * crcp[0], v[i][1] * crcp[1], v[i][2] * crcp[2], v[i][3] * crcp[3]);
-      const uint32_t hi = cvt4_e4m3(v[i][4] * crcp[4], v[i][5] * crcp[5], v[i][6] * crcp[6], v[i][7] * crcp[7]);
+      f.fence_row(i);
+      const uint32_t lo = cvt4_e4m3(f.get(i, 0) * crcp[0], f.get(i, 1) * crcp[1], f.get(i, 2) * crcp[2], f.get(i, 3) * crcp[3]);
+      const uint32_t hi = cvt4_e4m3(f.get(i, 4) * crcp[4], f.get(i, 5) * crcp[5], f.get(i, 6) * crcp[6], f.get(i, 7) * crcp[7]);
       if (row0 + i < p.M) {
         uint8_t* dst = bb + (row0 + i) * p.N + col0;
         if (p.vec_out) {
@@ -218,8 +259,8 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float r = crcp[j];
-      const uint32_t lo = cvt4_e4m3(v[0][j] * r, v[1][j] * r, v[2][j] * r, v[3][j] * r);
-      const uint32_t hi = cvt4_e4m3(v[4][j] * r, v[5][j] * r, v[6][j] * r, v[7][j] * r);
+      const uint32_t lo = cvt4_e4m3(f.get(0, j) * r, f.get(1, j) * r, f.get(2, j) * r, f.get(3, j) * r);
+      const uint32_t hi = cvt4_e4m3(f.get(4, j) * r, f.get(5, j) * r, f.get(6, j) * r, f.get(7, j) * r);
       const int n = cc * 8 + j;
       const int chunk = (rg >> 1) ^ ((n >> 3) & 7);
       *reinterpret_cast<uint2*>(&s_t[n * 128 + chunk * 16 + (rg & 1) * 8]) = make_uint2(lo, hi);
