@@ -99,6 +99,44 @@ __device__ __forceinline__ void store_pairs_bf16(const v16f& a, __amdgpu_buffer_
     __builtin_amdgcn_raw_buffer_store_b32((int)w, out, voff, s, 0);
   }
 }
+// bf16 through a per-wave LDS staging tile (32 rows x 64 B): the accumulator layout (a lane owns
+// one column) is turned into rows, so that every lane stores 16 contiguous bytes and one store
+// instruction covers 16 rows x 64 B.  The memory pipeline spends the same time on a 4-byte and a
+// 16-byte store instruction, so this is a quarter of the store issue time of store_pairs_bf16.
+// Only this wave touches its staging tile, so a counter wait between the phases is enough.
+// voff: lane's byte offset (row lane/4, 16-byte chunk lane%4) or kOob; soff: tile row 0, column 0.
+__device__ __forceinline__ void store_staged_bf16(const v16f& a, __amdgpu_buffer_rsrc_t out, uint8_t* stg, uint32_t voff,
+                                                  uint32_t soff, uint32_t pitch, bool accumulate, int lane) {
+  const bool odd = lane & 1;
+  uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 64 + ((lane & 31) >> 1) * 4;
+#pragma unroll
+  for (int v = 0; v < 16; v += 2) {
+    const float x0 = a[v], x1 = a[v + 1];
+    const float send = odd ? x0 : x1;
+    const float recv = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send), 0xB1, 0xF, 0xF, false));
+    const uint32_t w = odd ? pack2_bf16(recv, x1) : pack2_bf16(x0, recv);
+    *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = w;
+  }
+  // the reads below alias the writes above: keep the compiler from reordering them and let the
+  // writes land first
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  const uint8_t* rd = stg + (lane >> 2) * 64 + (lane & 3) * 16;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    v4i w = *(const v4i*)(rd + h * 1024);
+    const uint32_t s = soff + h * 16 * pitch;
+    if (accumulate) {
+      const v4i old = __builtin_amdgcn_raw_buffer_load_b128(out, voff, s, 0);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        w[q] = (int)pack2_bf16(bf16_lo((uint32_t)old[q]) + bf16_lo((uint32_t)w[q]), bf16_hi((uint32_t)old[q]) + bf16_hi((uint32_t)w[q]));
+    }
+    __builtin_amdgcn_raw_buffer_store_b128(w, out, voff, s, 0);
+    // A 16-byte store reads its data registers for a few cycles after it issues; the compiler
+    // only guards that window for stores without a scalar offset, so hold the registers here.
+    asm volatile("s_nop 4" ::"v"(w) : "memory");
+  }
+}
 __device__ __forceinline__ void store_single_bf16(const v16f& a, __amdgpu_buffer_rsrc_t out, uint32_t voff, uint32_t soff,
                                                   uint32_t pitch, bool accumulate) {
 #pragma unroll
@@ -253,6 +291,8 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   const uint32_t esz = p.out_dtype == PT_F32 ? 4 : 2;
   const uint32_t pitch = (uint32_t)p.ldo * esz;
   const bool pair_ok = p.out_dtype != PT_F32 && (p.ldo & 1) == 0 && (((uintptr_t)p.out) & 3) == 0;
+  const bool wide_ok = p.out_dtype != PT_F32 && (p.ldo & 7) == 0 && (((uintptr_t)p.out) & 15) == 0 &&
+                       (MODE != GEMM_K_GROUPED || (p.out_stride_g & 7) == 0);
 
   // ---- loader: walks (tile, 128-block) pairs ahead of the MFMAs and keeps the LDS ring full ----
   Tile L;
@@ -430,7 +470,19 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
     const __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(outp, 0, (int)((uint32_t)C.a_lim * pitch), kRsrcFlags);
     const uint32_t s_tile = (uint32_t)(C.a_row0 + wm0) * pitch + (uint32_t)(C.b_row0 + wn0) * esz;
     const int colw = C.b_row0 + wn0 + (lane & 31);
-    if (p.out_dtype != PT_F32 && pair_ok && (C.b_lim & 1) == 0) {
+    if (p.out_dtype != PT_F32 && wide_ok && (C.b_lim & 7) == 0) {
+      uint8_t* stg = lds + NS * STAGE + SC_RING * (BM + BN) * 4 + 512 + wave * 2048;
+      // rows first, then the column blocks of a row band back to back: adjacent 64-byte halves of
+      // a cache line are written by consecutive instructions
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int colc = C.b_row0 + wn0 + j * 32 + (lane & 3) * 8;
+          const uint32_t voff = colc < C.b_lim ? (uint32_t)(lane >> 2) * pitch + (uint32_t)(lane & 3) * 16 : kOob;
+          store_staged_bf16(acc[i][j], rs_out, stg, voff, s_tile + i * 32 * pitch + j * 64, pitch, ACC, lane);
+        }
+    } else if (p.out_dtype != PT_F32 && pair_ok && (C.b_lim & 1) == 0) {
       const bool odd = lane & 1;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
@@ -462,7 +514,7 @@ static int g_num_cus = 0;
 template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC>
 static int launch_one(GemmArgs a, hipStream_t stream) {
   constexpr int threads = WGM * WGN * 64;
-  constexpr size_t lds = (size_t)2 * (BM + BN) * 128 + 2 * (BM + BN) * 4 + 512;
+  constexpr size_t lds = (size_t)2 * (BM + BN) * 128 + 2 * (BM + BN) * 4 + 512 + (size_t)WGM * WGN * 2048;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)fp8_gemm_nt_persistent_kernel<MODE, BM, BN, WGM, WGN, ACC>,
