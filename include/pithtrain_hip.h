@@ -49,6 +49,16 @@ int pt_quant_rowwise_colwise(const void* x, int dtype, int64_t M, int64_t N, int
                              int ch_layout, const int32_t* offs, int32_t num_groups,
                              pt_stream_t stream);
 
+/* pt_quant_rowwise_colwise on gathered rows: output row r is quantised from source row
+ * row_index[r] of x (a negative index gives an all-zero row: zero bytes, the scale of amax 0).
+ * M counts output rows.  With row_index = the scatter's source map this is
+ * fp8cast_rowwise_colwise(scatter_for_grouped_gemm(x)) without materialising the permuted bf16
+ * copy (token_scatter.py:103-153 followed by deepgemm_quantize.py:204-259). */
+int pt_quant_rowwise_colwise_rows(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
+                                  const int32_t* row_index, void* tok_fp8, float* tok_scale,
+                                  void* ch_fp8, float* ch_scale, int ch_layout,
+                                  const int32_t* offs, int32_t num_groups, pt_stream_t stream);
+
 /* rowwise(x) + rowwise(x^T): t_fp8[N,M], t_scale[N,ceil(M/128)].
  * fp8cast_rowwise_transpose, deepgemm_quantize.py:429-482 */
 int pt_quant_rowwise_transpose(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
@@ -89,6 +99,17 @@ int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const void* b_fp8,
 int pt_gemm_m_grouped_nt(const void* a_fp8, const float* a_scale, const void* b_fp8,
                          const float* b_scale, void* out, int out_dtype, const int32_t* offs,
                          int32_t num_groups, int64_t M, int64_t N, int64_t K, pt_stream_t stream);
+
+/* pt_gemm_m_grouped_nt whose result row r is written to out[out_row_index[r], :] (negative
+ * index: the row is dropped); out is bf16 [out_rows, N], N % 8 == 0.  With out_row_index = the
+ * scatter's source map this is padded_index_gather(gemm(...), reverse) - the un-permute of
+ * token_scatter.py:297-309 (forward) or ScatterForGroupedGemm.backward (:271-284, dgrad) -
+ * without the intermediate [M, N] tensor. */
+int pt_gemm_m_grouped_nt_scatter(const void* a_fp8, const float* a_scale, const void* b_fp8,
+                                 const float* b_scale, void* out, int out_dtype,
+                                 const int32_t* offs, int32_t num_groups, int64_t M, int64_t N,
+                                 int64_t K, const int32_t* out_row_index, int64_t out_rows,
+                                 pt_stream_t stream);
 
 /* dW[g][n,k] = sum_{m in group g} dY[m,n] X[m,k] with colwise-quantised operands stored
  * transposed: dy_t[N,M] and x_t[K,M] (PT_CH_TRANSPOSED) and their scales dy_scale[M/128,N],

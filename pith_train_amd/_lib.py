@@ -27,11 +27,13 @@ SIGNATURES = {
     "pt_last_error": (c_char_p, []),
     "pt_abi_version": (c_int, []),
     "pt_quant_rowwise_colwise": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, c_int, P, I32, P]),
+    "pt_quant_rowwise_colwise_rows": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, P, c_int, P, I32, P]),
     "pt_quant_rowwise_transpose": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, P]),
     "pt_quant_rowwise_blockwise_transpose": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, P]),
     "pt_quant_blockwise_transpose_batched": (c_int, [P, c_int, I64, I64, I64, I64, I64, P, P, P, P, P]),
     "pt_gemm_nt_dense": (c_int, [P, P, P, P, P, c_int, I64, I64, I64, P]),
     "pt_gemm_m_grouped_nt": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P]),
+    "pt_gemm_m_grouped_nt_scatter": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, I64, P]),
     "pt_gemm_k_grouped_wgrad": (c_int, [P, P, P, P, P, c_int, c_int, P, I32, I64, I64, I64, P]),
     "pt_group_rows_workspace_bytes": (I64, [I64, I32]),
     "pt_group_rows": (c_int, [P, I64, I32, I32, P, P, P, P, I64, P, I64, P]),

@@ -280,6 +280,7 @@ static int dispatch_gemm(const GemmArgs& g, hipStream_t stream) {
   const int64_t lim = (1ll << 31) - 1;
   const bool fits = g.a_bytes < lim && g.b_bytes < lim && g.sa_bytes < lim && g.sb_bytes < lim && g.rows_a < lim &&
                     g.rows_b < lim && g.red < lim;
+  PT_REQUIRE(!g.out_row_index || (impl >= 0 && fits), "gemm: scattered output rows need the persistent kernel");
   if (impl < 0 || !fits) return launch_gemm<128, 128, 2, 2>(g, stream);
   return launch_gemm_persistent(g, impl, stream);
 }
@@ -310,9 +311,9 @@ extern "C" int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const v
   return dispatch_gemm(g, (hipStream_t)stream);
 }
 
-extern "C" int pt_gemm_m_grouped_nt(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
-                                    void* out, int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N, int64_t K,
-                                    pt_stream_t stream) {
+static int gemm_m_grouped_impl(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale, void* out,
+                               int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N, int64_t K,
+                               const int32_t* out_row_index, int64_t out_rows, pt_stream_t stream) {
   PT_REQUIRE(M >= 0 && N >= 0 && K >= 0 && G > 0, "gemm_m_grouped_nt: bad sizes");
   if (M == 0 || N == 0) return PT_OK;
   PT_REQUIRE(M % 128 == 0, "gemm_m_grouped_nt: M=%lld must be a multiple of 128", (long long)M);
@@ -331,7 +332,25 @@ extern "C" int pt_gemm_m_grouped_nt(const void* a_fp8, const float* a_scale, con
   g.a_bytes = M * K; g.b_bytes = N * K; g.sa_bytes = M * KB * 4; g.sb_bytes = NB * KB * 4;
   g.tiles_a = (int)(M / 128); g.tiles_b = (int)NB;
   g.total_tiles = (int64_t)g.tiles_a * g.tiles_b;
+  if (out_row_index) {
+    PT_REQUIRE(out_rows >= 0 && N % 8 == 0 && al16(out) && out_rows * N * 2 < (1ll << 32),
+               "gemm_m_grouped_nt_scatter: needs N %% 8 == 0, a 16-byte aligned output smaller than 4 GiB");
+    g.out_row_index = out_row_index; g.out_rows = out_rows;
+  }
   return dispatch_gemm(g, (hipStream_t)stream);
+}
+
+extern "C" int pt_gemm_m_grouped_nt(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
+                                    void* out, int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N, int64_t K,
+                                    pt_stream_t stream) {
+  return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, nullptr, 0, stream);
+}
+
+extern "C" int pt_gemm_m_grouped_nt_scatter(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
+                                            void* out, int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N,
+                                            int64_t K, const int32_t* out_row_index, int64_t out_rows, pt_stream_t stream) {
+  PT_REQUIRE(out_row_index, "gemm_m_grouped_nt_scatter: null out_row_index");
+  return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, out_row_index, out_rows, stream);
 }
 
 extern "C" int pt_gemm_k_grouped_wgrad(const void* dy_t_fp8, const float* dy_scale, const void* x_t_fp8, const float* x_scale,

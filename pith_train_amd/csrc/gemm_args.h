@@ -21,6 +21,8 @@ struct GemmArgs {
   int64_t a_bytes, b_bytes, sa_bytes, sb_bytes;  // extents of a, one group of b, and their scale arrays
   int64_t total_tiles;
   int pf_dist;                            // L2 prefetch distance in 128-blocks beyond the LDS ring
+  const int32_t* out_row_index;           // m-grouped only: output row of result row r (negative: dropped); null = identity
+  int64_t out_rows;                       // rows of the output when out_row_index is given
 };
 
 

@@ -137,6 +137,30 @@ __device__ __forceinline__ void store_staged_bf16(const v16f& a, __amdgpu_buffer
     asm volatile("s_nop 4" ::"v"(w) : "memory");
   }
 }
+// As store_staged_bf16 with an arbitrary output row per lane: voff0 / voff1 are the lane's byte
+// offsets (row start + 16-byte chunk, or kOob) for tile rows lane/4 and 16 + lane/4; soff the
+// column offset in bytes.
+__device__ __forceinline__ void store_staged_bf16_rows(const v16f& a, __amdgpu_buffer_rsrc_t out, uint8_t* stg, uint32_t voff0,
+                                                       uint32_t voff1, uint32_t soff, int lane) {
+  const bool odd = lane & 1;
+  uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 64 + ((lane & 31) >> 1) * 4;
+#pragma unroll
+  for (int v = 0; v < 16; v += 2) {
+    const float x0 = a[v], x1 = a[v + 1];
+    const float send = odd ? x0 : x1;
+    const float recv = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send), 0xB1, 0xF, 0xF, false));
+    const uint32_t w = odd ? pack2_bf16(recv, x1) : pack2_bf16(x0, recv);
+    *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = w;
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  const uint8_t* rd = stg + (lane >> 2) * 64 + (lane & 3) * 16;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const v4i w = *(const v4i*)(rd + h * 1024);
+    __builtin_amdgcn_raw_buffer_store_b128(w, out, h ? voff1 : voff0, soff, 0);
+    asm volatile("s_nop 4" ::"v"(w) : "memory");  // see store_staged_bf16
+  }
+}
 __device__ __forceinline__ void store_single_bf16(const v16f& a, __amdgpu_buffer_rsrc_t out, uint32_t voff, uint32_t soff,
                                                   uint32_t pitch, bool accumulate) {
 #pragma unroll
@@ -470,7 +494,29 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
     const __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(outp, 0, (int)((uint32_t)C.a_lim * pitch), kRsrcFlags);
     const uint32_t s_tile = (uint32_t)(C.a_row0 + wm0) * pitch + (uint32_t)(C.b_row0 + wn0) * esz;
     const int colw = C.b_row0 + wn0 + (lane & 31);
-    if (p.out_dtype != PT_F32 && wide_ok && (C.b_lim & 7) == 0) {
+    if (MODE == GEMM_M_GROUPED && p.out_row_index) {
+      // Result row r goes to output row out_row_index[r] (the un-permute folded into the store);
+      // rows of the group's padding map to a negative index and are dropped.
+      uint8_t* stg = lds + NS * STAGE + SC_RING * (BM + BN) * 4 + 512 + wave * 2048;
+      const __amdgpu_buffer_rsrc_t rs_sc = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, (int)((uint32_t)p.out_rows * pitch), kRsrcFlags);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        uint32_t vrow[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int r = C.a_row0 + wm0 + i * 32 + h * 16 + (lane >> 2);
+          const int dst = r < C.a_lim ? p.out_row_index[r] : -1;
+          vrow[h] = dst >= 0 ? (uint32_t)dst * pitch + (uint32_t)(lane & 3) * 16 : kOob;
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int colc = C.b_row0 + wn0 + j * 32 + (lane & 3) * 8;
+          const bool col_ok = colc < C.b_lim;
+          store_staged_bf16_rows(acc[i][j], rs_sc, stg, col_ok ? vrow[0] : kOob, col_ok ? vrow[1] : kOob,
+                                 (uint32_t)(C.b_row0 + wn0 + j * 32) * 2, lane);
+        }
+      }
+    } else if (p.out_dtype != PT_F32 && wide_ok && (C.b_lim & 7) == 0) {
       uint8_t* stg = lds + NS * STAGE + SC_RING * (BM + BN) * 4 + 512 + wave * 2048;
       // rows first, then the column blocks of a row band back to back: adjacent 64-byte halves of
       // a cache line are written by consecutive instructions

@@ -29,6 +29,7 @@ struct QuantArgs {
   int32_t vec_in;     // 16-byte loads legal (alignment + N % 8 == 0)
   int32_t vec_out;    // 8-byte row-major stores legal (N % 8 == 0)
   int32_t vec_out_t;  // 16-byte transposed stores legal
+  const int32_t* row_index;  // optional [M]: source row of output row r (negative: a zero row); null = identity
 };
 
 template <typename T> struct Loader;
@@ -118,16 +119,20 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
     const bool col_ok = col0 < p.N;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      if (col_ok && row0 + i < p.M) f.load_row(i, xb + ((row0 + i) * p.ldx + col0) * Loader<T>::kBytes);
+      int64_t sr = row0 + i;
+      if (p.row_index && sr < p.M) sr = p.row_index[sr];
+      if (col_ok && row0 + i < p.M && sr >= 0) f.load_row(i, xb + (sr * p.ldx + col0) * Loader<T>::kBytes);
       else f.zero_row(i);
     }
   } else {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       f.zero_row(i);
+      int64_t sr = row0 + i;
+      if (p.row_index && sr < p.M) sr = p.row_index[sr];
 #pragma unroll
       for (int j = 0; j < 8; ++j)
-        if (row0 + i < p.M && col0 + j < p.N) f.set(i, j, xb + ((row0 + i) * p.ldx + col0 + j) * Loader<T>::kBytes);
+        if (row0 + i < p.M && sr >= 0 && col0 + j < p.N) f.set(i, j, xb + (sr * p.ldx + col0 + j) * Loader<T>::kBytes);
     }
   }
 
@@ -325,7 +330,7 @@ static void fill_common(QuantArgs& a, const void* x, int dtype, int64_t M, int64
   a.x = x; a.M = M; a.N = N; a.ldx = ldx; a.x_stride_g = 0;
   a.a_stride_g = 0; a.a_scale_stride_g = 0; a.b_stride_g = 0; a.b_scale_stride_g = 0;
   a.tiles_m = (int32_t)cdiv(M, 128); a.tiles_n = (int32_t)cdiv(N, 128);
-  a.offs = nullptr; a.num_groups = 0;
+  a.offs = nullptr; a.num_groups = 0; a.row_index = nullptr;
   const int eb = dtype == PT_F32 ? 4 : 2;
   a.vec_in = (N % 8 == 0) && ((ldx * eb) % 16 == 0) && (((uintptr_t)x) % 16 == 0);
   a.vec_out = (N % 8 == 0);
@@ -336,10 +341,30 @@ static void fill_common(QuantArgs& a, const void* x, int dtype, int64_t M, int64
 
 using namespace pt;
 
+static int quant_rowwise_colwise_impl(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx, const int32_t* row_index,
+                                      void* tok_fp8, float* tok_scale, void* ch_fp8, float* ch_scale, int ch_layout,
+                                      const int32_t* offs, int32_t num_groups, pt_stream_t stream);
+
 extern "C" int pt_quant_rowwise_colwise(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
                                         void* tok_fp8, float* tok_scale, void* ch_fp8,
                                         float* ch_scale, int ch_layout, const int32_t* offs,
                                         int32_t num_groups, pt_stream_t stream) {
+  return quant_rowwise_colwise_impl(x, dtype, M, N, ldx, nullptr, tok_fp8, tok_scale, ch_fp8, ch_scale, ch_layout, offs,
+                                    num_groups, stream);
+}
+
+extern "C" int pt_quant_rowwise_colwise_rows(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
+                                             const int32_t* row_index, void* tok_fp8, float* tok_scale,
+                                             void* ch_fp8, float* ch_scale, int ch_layout,
+                                             const int32_t* offs, int32_t num_groups, pt_stream_t stream) {
+  PT_REQUIRE(row_index || M == 0, "quant_rowwise_colwise_rows: null row_index");
+  return quant_rowwise_colwise_impl(x, dtype, M, N, ldx, row_index, tok_fp8, tok_scale, ch_fp8, ch_scale, ch_layout, offs,
+                                    num_groups, stream);
+}
+
+static int quant_rowwise_colwise_impl(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx, const int32_t* row_index,
+                                      void* tok_fp8, float* tok_scale, void* ch_fp8, float* ch_scale, int ch_layout,
+                                      const int32_t* offs, int32_t num_groups, pt_stream_t stream) {
   PT_REQUIRE(M >= 0 && N >= 0 && M % 128 == 0, "quant_rowwise_colwise: M=%lld must be a multiple of 128", (long long)M);
   PT_REQUIRE(ldx >= N, "quant_rowwise_colwise: ldx < N");
   if (M == 0 || N == 0) return PT_OK;
@@ -347,6 +372,7 @@ extern "C" int pt_quant_rowwise_colwise(const void* x, int dtype, int64_t M, int
   QuantArgs a;
   fill_common(a, x, dtype, M, N, ldx);
   a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)ch_fp8; a.b_scale = ch_scale;
+  a.row_index = row_index;
   hipStream_t s = (hipStream_t)stream;
   switch (ch_layout) {
     case PT_CH_ROWMAJOR:   return launch_quant<A_ROW, B_COL, BL_ROWMAJOR, BS_MB_N>(a, dtype, 1, s);

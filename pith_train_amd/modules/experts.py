@@ -22,11 +22,12 @@ import torch.nn as nn
 from ..dualpipe_utils import FP8WeightCacheControl
 from ..operators.clamped_swiglu import clamped_swiglu
 from ..operators.deepgemm_quantize import fp8cast_blockwise_transpose_batched
-from ..operators.grouped_linear import FP8GroupedLinearFunc, GroupedLinearFunc
+from ..operators.grouped_linear import FP8GroupedLinear, FP8GroupedLinearFunc, GroupedLinearFunc
 from ..operators.indexed_bias_add import indexed_bias_add
 from ..operators.silu_mul import silu_mul, silu_mul_halves
 from ..operators.token_scatter import (
     group_indices,
+    group_rows_with_sizes,
     padded_index_gather,
     precompute_group_indices,
     scatter_for_grouped_gemm,
@@ -41,9 +42,16 @@ class Qwen3MoeExperts(nn.Module):
         self.up_proj = training.GroupedLinear(num_experts, hidden_size, moe_intermediate_size)
         self.down_proj = training.GroupedLinear(num_experts, moe_intermediate_size, hidden_size)
 
-    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None):
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None):
+        """``row_map`` (extension, FP8 layers only): the scatter's int32 source-row map.  ``x`` is
+        then the un-permuted ``[m, H]`` token tensor and the result comes back un-permuted; the
+        permutation happens inside the first quantisation and the last GEMM's store."""
         gi = precompute_group_indices(grouped_mm_offs, x.shape[0])
         kwargs = dict(grouped_mm_offs=grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, group_indices=gi)
+        if row_map is not None:
+            g = self.gate_proj(x, in_rows=row_map, **kwargs)
+            u = self.up_proj(x, in_rows=row_map, **kwargs)
+            return self.down_proj(silu_mul(g, u), out_rows=row_map, out_m=x.shape[0], **kwargs)
         g = self.gate_proj(x, **kwargs)
         u = self.up_proj(x, **kwargs)
         return self.down_proj(silu_mul(g, u), **kwargs)
@@ -75,9 +83,13 @@ class Qwen35MoeExperts(nn.Module):
         self.gate_up_proj = training.GroupedLinear(num_experts, hidden_size, 2 * moe_intermediate_size)
         self.down_proj = training.GroupedLinear(num_experts, moe_intermediate_size, hidden_size)
 
-    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None):
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None):
+        """``row_map``: see :meth:`Qwen3MoeExperts.forward`."""
         gi = precompute_group_indices(grouped_mm_offs, x.shape[0])
         kwargs = dict(grouped_mm_offs=grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, group_indices=gi)
+        if row_map is not None:
+            gate_up = self.gate_up_proj(x, in_rows=row_map, **kwargs)
+            return self.down_proj(silu_mul_halves(gate_up), out_rows=row_map, out_m=x.shape[0], **kwargs)
         gate_up = self.gate_up_proj(x, **kwargs)
         # the halves are read in place (same arithmetic as silu_mul on contiguous copies)
         return self.down_proj(silu_mul_halves(gate_up), **kwargs)
@@ -126,14 +138,27 @@ class GptOssExperts(nn.Module):
 
 
 def forward_stage3(experts: nn.Module, gathered_tokens, expert_idxs, experts_per_rank: int, expand_idx=None,
-                   fuse_expand: bool = True):
+                   fuse_expand: bool = True, fuse_permute: bool = True):
     """Expert compute between the dispatch and combine all-to-alls.
+
+    With ``fuse_permute`` (FP8 Qwen3 / DeepSeek / Qwen3.5 experts, no ``expand_idx``) the permuted
+    copy of the tokens, its inverse gather and their two backward passes are never materialised:
+    only the index half of the scatter runs, the first quantisation reads rows through the
+    source map and the last GEMM of forward and of backward stores rows through it.  The result
+    is bit-identical to the unfused composition.
 
     ``expand_idx`` (EP > 1) re-expands the deduplicated received rows to one row per routed
     (token, expert) pair.  With ``fuse_expand`` that gather is folded into the scatter's row copy
     (each unique row is read once per use and no expanded copy is materialised); without it the
     two steps run separately as in the reference.
     """
+    if (fuse_permute and expand_idx is None and training.fp8 and expert_idxs.shape[0] > 0
+            and isinstance(experts, (Qwen3MoeExperts, Qwen35MoeExperts))
+            and isinstance(experts.down_proj, FP8GroupedLinear)
+            and experts.down_proj.out_features % 8 == 0 and experts.down_proj.in_features % 8 == 0):
+        _, grouped_mm_offs, ks, ks_tensor, src_of = group_rows_with_sizes(
+            expert_idxs, experts_per_rank, device=gathered_tokens.device)
+        return experts(gathered_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, row_map=src_of)
     pre = None
     if expand_idx is not None:
         if fuse_expand:

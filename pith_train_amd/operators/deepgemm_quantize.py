@@ -20,6 +20,7 @@ __all__ = [
     "fp8cast_blockwise_transpose",
     "fp8cast_blockwise_transpose_batched",
     "fp8cast_rowwise_colwise_t",
+    "fp8cast_rowwise_colwise_t_rows",
 ]
 
 FP8 = torch.float8_e4m3fn
@@ -70,6 +71,30 @@ def _rowwise_colwise(x: torch.Tensor, layout: int, offs: torch.Tensor | None):
 def fp8cast_rowwise_colwise(x: torch.Tensor):
     """(tok_fp8[M,N], tok_scale[M,ceil(N/128)], ch_fp8[M,N], ch_scale[M//128,N]); M % 128 == 0."""
     return _rowwise_colwise(x, _lib.PT_CH_ROWMAJOR, None)
+
+
+def fp8cast_rowwise_colwise_t_rows(x: torch.Tensor, row_index: torch.Tensor):
+    """:func:`fp8cast_rowwise_colwise_t` of ``x[row_index]`` (rows with a negative index are zero)
+    without materialising the gathered tensor.  ``row_index`` is int32 ``[M]``, ``M % 128 == 0``."""
+    assert x.ndim == 2 and row_index.ndim == 1 and row_index.dtype == torch.int32
+    assert row_index.shape[0] % 128 == 0, f"row count {row_index.shape[0]} must be a multiple of 128"
+    x = _prep2d(x)
+    _lib.require_cuda(row_index)
+    row_index = row_index.contiguous()
+    M, N = row_index.shape[0], x.shape[1]
+    dev = x.device
+    out_tok = torch.empty((M, N), dtype=FP8, device=dev)
+    scale_tok = torch.empty((M, _cdiv(N, 128)), dtype=torch.float32, device=dev)
+    out_ch = torch.empty((N, M), dtype=FP8, device=dev)
+    scale_ch = torch.empty((M // 128, N), dtype=torch.float32, device=dev)
+    if M and N:
+        ld = x.stride(0) if x.shape[0] > 1 else N
+        _lib.call(
+            "pt_quant_rowwise_colwise_rows", x.data_ptr(), _lib.dtype_code(x.dtype), M, N, ld,
+            row_index.data_ptr(), out_tok.data_ptr(), scale_tok.data_ptr(), out_ch.data_ptr(),
+            scale_ch.data_ptr(), _lib.PT_CH_TRANSPOSED, None, 0, _lib.stream_ptr(dev),
+        )  # fmt: skip
+    return out_tok, scale_tok, out_ch, scale_ch
 
 
 def fp8cast_rowwise_colwise_t(x: torch.Tensor):

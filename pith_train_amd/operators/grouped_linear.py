@@ -24,7 +24,11 @@ import torch.nn.functional as F
 
 from .. import _lib
 from ..dualpipe_utils import FP8WeightCacheControl, WeightGradStore
-from .deepgemm_quantize import fp8cast_blockwise_transpose_batched, fp8cast_rowwise_colwise_t
+from .deepgemm_quantize import (
+    fp8cast_blockwise_transpose_batched,
+    fp8cast_rowwise_colwise_t,
+    fp8cast_rowwise_colwise_t_rows,
+)
 
 
 def _grouped_mm(a: torch.Tensor, b: torch.Tensor, offs: torch.Tensor) -> torch.Tensor:
@@ -101,12 +105,22 @@ class GroupedLinear(nn.Module):
 # ------------------------------------------------------------------------------------------------
 # FP8
 # ------------------------------------------------------------------------------------------------
-def m_grouped_fp8_gemm_nt(a, b, out: torch.Tensor, grouped_mm_offs: torch.Tensor) -> torch.Tensor:
+def m_grouped_fp8_gemm_nt(a, b, out: torch.Tensor, grouped_mm_offs: torch.Tensor,
+                          out_rows: torch.Tensor | None = None) -> torch.Tensor:
     """out[rows_g] = a[rows_g] @ b[g].T with a=(fp8[M,K], scale[M,K/128]), b=(fp8[G,N,K],
-    scale[G,N/128,K/128]).  Rows at or past ``grouped_mm_offs[-1]`` are left untouched."""
+    scale[G,N/128,K/128]).  Rows at or past ``grouped_mm_offs[-1]`` are left untouched.  With
+    ``out_rows`` (int32 [M]) result row r is written to ``out[out_rows[r]]`` instead (negative:
+    dropped)."""
     (a_fp8, a_s), (b_fp8, b_s) = a, b
     M, K = a_fp8.shape
     G, N, _ = b_fp8.shape
+    if out_rows is not None:
+        _lib.call(
+            "pt_gemm_m_grouped_nt_scatter", a_fp8.data_ptr(), a_s.data_ptr(), b_fp8.data_ptr(),
+            b_s.data_ptr(), out.data_ptr(), _lib.dtype_code(out.dtype), grouped_mm_offs.data_ptr(), G,
+            M, N, K, out_rows.data_ptr(), out.shape[0], _lib.stream_ptr(out.device),
+        )  # fmt: skip
+        return out
     _lib.call(
         "pt_gemm_m_grouped_nt", a_fp8.data_ptr(), a_s.data_ptr(), b_fp8.data_ptr(), b_s.data_ptr(),
         out.data_ptr(), _lib.dtype_code(out.dtype), grouped_mm_offs.data_ptr(), G, M, N, K,
@@ -144,33 +158,58 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
         ks_tensor: torch.Tensor,
         quantized_weight: tuple,
         group_indices: torch.Tensor | None = None,
+        in_rows: torch.Tensor | None = None,
+        out_rows: torch.Tensor | None = None,
+        out_m: int | None = None,
     ):
+        """``in_rows`` / ``out_rows`` (extension; int32 ``[M]`` source-row maps as produced by the
+        scatter, every non-negative value occurring once) fold the token permutation into this
+        layer: with ``in_rows`` the input is the un-permuted ``[m, K]`` tensor and grouped row r is
+        read from ``input[in_rows[r]]``; with ``out_rows`` the result is returned un-permuted
+        (``[out_m, N]``, row ``out_rows[r]`` holding grouped row r).  Backward mirrors both."""
         weight_fp8, scale_weight, weight_t_fp8, scale_weight_t = quantized_weight
-        M, K = input.shape
-        num_groups, N, _ = weight.shape
-        input_fp8, scale_input, input_ch_t, scale_input_ch = fp8cast_rowwise_colwise_t(input)
-        output = torch.empty((M, N), device=input.device, dtype=input.dtype)
+        num_groups, N, K = weight.shape
+        if in_rows is not None:
+            M = in_rows.shape[0]
+            input_fp8, scale_input, input_ch_t, scale_input_ch = fp8cast_rowwise_colwise_t_rows(input, in_rows)
+        else:
+            M = input.shape[0]
+            input_fp8, scale_input, input_ch_t, scale_input_ch = fp8cast_rowwise_colwise_t(input)
+        if out_rows is not None:
+            assert out_m is not None, "out_rows needs out_m, the row count of the un-permuted result"
+            output = torch.empty((out_m, N), device=input.device, dtype=input.dtype)
+        else:
+            output = torch.empty((M, N), device=input.device, dtype=input.dtype)
         m_grouped_fp8_gemm_nt(
-            (input_fp8, scale_input), (weight_fp8, scale_weight), output, grouped_mm_offs
+            (input_fp8, scale_input), (weight_fp8, scale_weight), output, grouped_mm_offs, out_rows
         )
         ctx.save_for_backward(
-            weight_t_fp8, scale_weight_t, grouped_mm_offs, input_ch_t, scale_input_ch, ks_tensor
+            weight_t_fp8, scale_weight_t, grouped_mm_offs, input_ch_t, scale_input_ch, ks_tensor,
+            in_rows, out_rows,
         )
         ctx.weight_ref = weight
         ctx.ks = ks
         ctx.dims = (M, K, N, num_groups)
+        ctx.in_m = input.shape[0]
         return output
 
     @staticmethod
     def backward(ctx, grad_output):
-        weight_t_fp8, scale_weight_t, offs, input_ch_t, scale_input_ch, ks_tensor = ctx.saved_tensors
+        (weight_t_fp8, scale_weight_t, offs, input_ch_t, scale_input_ch, ks_tensor, in_rows,
+         out_rows) = ctx.saved_tensors  # fmt: skip
         weight = ctx.weight_ref
         M, K, N, num_groups = ctx.dims
         grad_output = grad_output.contiguous()
-        grad_fp8, scale_grad, grad_ch_t, scale_grad_ch = fp8cast_rowwise_colwise_t(grad_output)
+        if out_rows is not None:  # the gradient arrives un-permuted: gather while quantising
+            grad_fp8, scale_grad, grad_ch_t, scale_grad_ch = fp8cast_rowwise_colwise_t_rows(grad_output, out_rows)
+        else:
+            grad_fp8, scale_grad, grad_ch_t, scale_grad_ch = fp8cast_rowwise_colwise_t(grad_output)
 
-        grad_input = torch.empty((M, K), device=grad_output.device, dtype=grad_output.dtype)
-        m_grouped_fp8_gemm_nt((grad_fp8, scale_grad), (weight_t_fp8, scale_weight_t), grad_input, offs)
+        rows_in = ctx.in_m if in_rows is not None else M
+        grad_input = torch.empty((rows_in, K), device=grad_output.device, dtype=grad_output.dtype)
+        m_grouped_fp8_gemm_nt(
+            (grad_fp8, scale_grad), (weight_t_fp8, scale_weight_t), grad_input, offs, in_rows
+        )
 
         def grad_weight_fn(a, b, offs):
             # bf16(sum) is formed in the GEMM epilogue; an existing grad is accumulated there too
@@ -198,7 +237,7 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
             )
         else:
             grad_weight_fn(a_wgrad, b_wgrad, offs)
-        return grad_input, None, None, None, None, None, None
+        return grad_input, None, None, None, None, None, None, None, None, None
 
 
 class FP8GroupedLinear(nn.Module):
@@ -232,10 +271,13 @@ class FP8GroupedLinear(nn.Module):
         ks: list | None = None,
         ks_tensor: torch.Tensor | None = None,
         group_indices: torch.Tensor | None = None,
+        in_rows: torch.Tensor | None = None,
+        out_rows: torch.Tensor | None = None,
+        out_m: int | None = None,
     ) -> torch.Tensor:
         if input.shape[0] == 0:
             return input @ self.weight[0].T  # keeps a grad_fn with zero rows
         return FP8GroupedLinearFunc.apply(
             input, self.weight, grouped_mm_offs, ks, ks_tensor, self._get_quantized_weight(),
-            group_indices,
+            group_indices, in_rows, out_rows, out_m,
         )  # fmt: skip

@@ -52,6 +52,25 @@ def group_rows(expert_idxs: torch.Tensor, num_groups: int, padding_alignment: in
     return reverse, offs, ks_tensor, src_of
 
 
+def group_rows_with_sizes(expert_idxs: torch.Tensor, num_groups: int, padding_alignment: int = 128, device=None):
+    """The index half of :func:`scatter_for_grouped_gemm` on its own: returns ``(reverse i64[m],
+    grouped_mm_offs i32[G], ks list[int], ks_tensor i32[G], src_of i32[sum(ks)])`` where
+    ``src_of[r]`` is the source row of grouped row r (-1 for a padding row).  No rows are moved."""
+    _lib.require_cuda(expert_idxs)
+    expert_idxs = expert_idxs.contiguous()
+    assert expert_idxs.dtype == torch.int64, "expert_idxs must be int64"
+    m = expert_idxs.shape[0]
+    dev = expert_idxs.device
+    max_m_padded = m + num_groups * (padding_alignment - 1)
+    max_m_padded = -(-max_m_padded // _GEMM_ALLOC_ALIGNMENT) * _GEMM_ALLOC_ALIGNMENT
+    reverse, offs, ks_tensor, src_of = group_rows(expert_idxs, num_groups, padding_alignment, max_m_padded)
+    ks_cpu = get_pinned_buffer("ks", num_groups, torch.int32)
+    ks_cpu.copy_(ks_tensor, non_blocking=True)
+    torch.cuda.current_stream(dev).synchronize()
+    ks = ks_cpu.tolist()
+    return reverse, offs, ks, ks_tensor, src_of[: sum(ks)]
+
+
 def permute_rows(input_tokens, src_of, out, offs_last, pre_index=None):
     """out[r] = input[src_of[r]] (optionally through ``pre_index``), zero where src_of[r] < 0."""
     H = input_tokens.shape[1]

@@ -68,8 +68,9 @@ CASES = [
 ]
 
 
+@pytest.mark.parametrize("fuse_permute", [True, False])
 @pytest.mark.parametrize("kind,E,H,I,T,k,zipf", CASES)
-def test_stage3_forward_backward(kind, E, H, I, T, k, zipf):
+def test_stage3_forward_backward(kind, E, H, I, T, k, zipf, fuse_permute):
     from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
     from pith_train_amd.modules.experts import forward_stage3
 
@@ -85,13 +86,40 @@ def test_stage3_forward_backward(kind, E, H, I, T, k, zipf):
     mod, params = _build(kind, E, H, I, w)
     FP8WeightCacheControl.step()
     tok = tokens.cuda().requires_grad_(True)
-    out = forward_stage3(mod, tok, expert_idxs.cuda(), E)
+    out = forward_stage3(mod, tok, expert_idxs.cuda(), E, fuse_permute=fuse_permute)
     _close(out, ref["out"], "out")
     out.backward(dy.cuda())
     _close(tok.grad, ref["grad_tokens"], "grad_tokens")
     for name, p in params.items():
         assert p.grad is not None and p.grad.dtype == torch.bfloat16, name
         _close(p.grad, ref[name], name)
+
+
+@pytest.mark.parametrize("kind,E,H,I,T,k,zipf", [c for c in CASES if c[0] != "gpt_oss"] + [("fused", 128, 256, 128, 2048, 8, 1.2)])
+def test_stage3_permute_folded_into_quant_and_gemm_is_bit_identical(kind, E, H, I, T, k, zipf):
+    """The path that never materialises the permuted tokens (rows gathered by the first
+    quantisation, scattered by the last GEMM store, forward and backward) gives the same bits as
+    scatter -> experts -> gather."""
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules.experts import forward_stage3
+
+    ids = OM.make_routing(T, E, k, seed=3, zipf_s=zipf)
+    g = torch.Generator().manual_seed(4)
+    tokens = torch.randn((T * k, H), generator=g).bfloat16().cuda()
+    dy = torch.randn((T * k, H), generator=g).bfloat16().cuda()
+    w = _weights(kind, E, H, I, 5)
+    res = []
+    for fuse in (True, False):
+        mod, params = _build(kind, E, H, I, w)
+        FP8WeightCacheControl.step()
+        tok = tokens.clone().requires_grad_(True)
+        out = forward_stage3(mod, tok, ids.reshape(-1).cuda(), E, fuse_permute=fuse)
+        out.backward(dy)
+        res.append((out.detach(), tok.grad, {n: p.grad for n, p in params.items()}))
+    assert torch.equal(res[0][0], res[1][0]), "forward output differs"
+    assert torch.equal(res[0][1], res[1][1]), "token gradient differs"
+    for n in res[0][2]:
+        assert torch.equal(res[0][2][n], res[1][2][n]), f"{n} gradient differs"
 
 
 def test_stage3_with_dedup_expand_fused_and_unfused():
