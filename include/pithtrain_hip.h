@@ -59,6 +59,22 @@ int pt_quant_rowwise_colwise_rows(const void* x, int dtype, int64_t M, int64_t N
                                   void* ch_fp8, float* ch_scale, int ch_layout,
                                   const int32_t* offs, int32_t num_groups, pt_stream_t stream);
 
+/* SwiGLU fused into the activation quantisation (bf16 only).  Forward: h = bf16(silu(gate) * up)
+ * with gate = gate_up[:, :half], up = gate_up[:, half:], quantised as pt_quant_rowwise_colwise
+ * with the PT_CH_TRANSPOSED twin: tok_fp8[M,half], tok_scale[M,ceil(half/128)], ch_t_fp8[half,M],
+ * ch_scale[M/128,half].  Same bits as silu_mul (silu_mul.py:28-49) followed by
+ * fp8cast_rowwise_colwise (deepgemm_quantize.py:204-259); h itself is never written. */
+int pt_silu_mul_quant_rowwise_colwise(const void* gate_up, int64_t M, int64_t half,
+                                      int64_t ld_gate_up, void* tok_fp8, float* tok_scale,
+                                      void* ch_t_fp8, float* ch_scale, pt_stream_t stream);
+/* Backward twin: [dgate | dup] = silu_mul backward (silu_mul.py:52-87) of grad_h[M,half] at the
+ * saved gate_up[M,2*half], rounded to bf16 and quantised to tok_fp8[M,2*half],
+ * tok_scale[M,ceil(2*half/128)], ch_t_fp8[2*half,M], ch_scale[M/128,2*half]. */
+int pt_silu_mul_bwd_quant_rowwise_colwise(const void* grad_h, int64_t ld_grad_h,
+                                          const void* gate_up, int64_t ld_gate_up, int64_t M,
+                                          int64_t half, void* tok_fp8, float* tok_scale,
+                                          void* ch_t_fp8, float* ch_scale, pt_stream_t stream);
+
 /* rowwise(x) + rowwise(x^T): t_fp8[N,M], t_scale[N,ceil(M/128)].
  * fp8cast_rowwise_transpose, deepgemm_quantize.py:429-482 */
 int pt_quant_rowwise_transpose(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,

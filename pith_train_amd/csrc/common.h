@@ -51,6 +51,23 @@ __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
   return r & 0xFFFFu;
 }
 
+// ---- SwiGLU arithmetic shared by the epilogue kernels and the fused activation + quantisation ----
+__device__ __forceinline__ float sigmoidf_fast(float x) {
+  return __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-x)));
+}
+
+// The arithmetic is spelled with explicit round-to-nearest operations so that every kernel that
+// uses it (flat and row-strided) produces the same bits whatever the compiler would contract.
+__device__ __forceinline__ float silu_mul_f(float g, float u) {
+  return __fmul_rn(__fmul_rn(g, sigmoidf_fast(g)), u);
+}
+__device__ __forceinline__ void silu_mul_b(float d, float g, float u, float& dg, float& du) {
+  const float sig = sigmoidf_fast(g);
+  const float silu = __fmul_rn(g, sig);
+  du = __fmul_rn(d, silu);
+  dg = __fmul_rn(__fmul_rn(__fmul_rn(d, u), sig), __fsub_rn(__fadd_rn(1.0f, g), silu));
+}
+
 // ---- storage types: 8-wide vector and scalar load/store with fp32 math ---------------------------
 struct st_bf16 {
   static constexpr int kBytes = 2;

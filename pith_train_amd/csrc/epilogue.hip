@@ -7,22 +7,8 @@
 
 namespace pt {
 
-__device__ __forceinline__ float sigmoidf_fast(float x) {
-  return __builtin_amdgcn_rcpf(__fadd_rn(1.0f, __expf(-x)));
-}
+// sigmoidf_fast / silu_mul_f / silu_mul_b live in common.h (shared with the fused quantisation).
 
-// ---- silu_mul ---------------------------------------------------------------------------------
-// The arithmetic is spelled with explicit round-to-nearest operations so that every kernel that
-// uses it (flat and row-strided) produces the same bits whatever the compiler would contract.
-__device__ __forceinline__ float silu_mul_f(float g, float u) {
-  return __fmul_rn(__fmul_rn(g, sigmoidf_fast(g)), u);
-}
-__device__ __forceinline__ void silu_mul_b(float d, float g, float u, float& dg, float& du) {
-  const float sig = sigmoidf_fast(g);
-  const float silu = __fmul_rn(g, sig);
-  du = __fmul_rn(d, silu);
-  dg = __fmul_rn(__fmul_rn(__fmul_rn(d, u), sig), __fsub_rn(__fadd_rn(1.0f, g), silu));
-}
 template <typename S>
 __global__ __launch_bounds__(256) void silu_mul_fwd_kernel(const char* gate, const char* up, char* out, int64_t n) {
   const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;

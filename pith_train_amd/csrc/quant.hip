@@ -30,6 +30,8 @@ struct QuantArgs {
   int32_t vec_out;    // 8-byte row-major stores legal (N % 8 == 0)
   int32_t vec_out_t;  // 16-byte transposed stores legal
   const int32_t* row_index;  // optional [M]: source row of output row r (negative: a zero row); null = identity
+  const void* x2; int64_t ldx2;  // fused SwiGLU backward: the saved gate_up [M, 2*half]
+  int64_t half;                  // fused SwiGLU: width of one half of gate_up
 };
 
 template <typename T> struct Loader;
@@ -97,7 +99,9 @@ template <> struct Frag<float> {
   __device__ __forceinline__ void fence_row(int) {}
 };
 
-template <typename T, int AM, int BMODE, int BL, int BS>
+enum { PRO_NONE = 0, PRO_SILU_FWD = 1, PRO_SILU_BWD = 2 };  // what the tile is computed from
+
+template <typename T, int AM, int BMODE, int BL, int BS, int PRO = PRO_NONE>
 __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   __shared__ float s_colmax[4][128];
   __shared__ float s_blk[4];
@@ -115,7 +119,44 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   const char* xb = reinterpret_cast<const char*>(p.x) + g * p.x_stride_g * Loader<T>::kBytes;
 
   Frag<T> f;
-  if (p.vec_in) {
+  if constexpr (PRO != PRO_NONE) {
+    // The quantised tensor is the bf16-rounded SwiGLU output (forward: h = silu(gate) * up from
+    // gate_up = x) or its gradient (backward: [dgate | dup] from grad_h = x and gate_up = x2),
+    // computed here instead of being written to memory and read back.  bf16 only, 16-byte loads.
+    const bool col_ok = col0 < p.N;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (col_ok && row0 + i < p.M) {
+        const int64_t r = row0 + i;
+        float g[8], u[8], o[8];
+        if (PRO == PRO_SILU_FWD) {
+          const char* gp = xb + (r * p.ldx + col0) * 2;
+          st_bf16::load8(gp, g);
+          st_bf16::load8(gp + p.half * 2, u);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) o[j] = silu_mul_f(g[j], u[j]);
+        } else {
+          const bool up_half = col0 >= p.half;
+          const int64_t cc = col0 - (up_half ? p.half : 0);
+          float d[8];
+          st_bf16::load8(xb + (r * p.ldx + cc) * 2, d);
+          const char* gp = (const char*)p.x2 + (r * p.ldx2 + cc) * 2;
+          st_bf16::load8(gp, g);
+          st_bf16::load8(gp + p.half * 2, u);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            float dg, du;
+            silu_mul_b(d[j], g[j], u[j], dg, du);
+            o[j] = up_half ? du : dg;
+          }
+        }
+        f.w[i][0] = pack_bf16x2(o[0], o[1]); f.w[i][1] = pack_bf16x2(o[2], o[3]);
+        f.w[i][2] = pack_bf16x2(o[4], o[5]); f.w[i][3] = pack_bf16x2(o[6], o[7]);
+      } else {
+        f.zero_row(i);
+      }
+    }
+  } else if (p.vec_in) {
     const bool col_ok = col0 < p.N;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -330,7 +371,7 @@ static void fill_common(QuantArgs& a, const void* x, int dtype, int64_t M, int64
   a.x = x; a.M = M; a.N = N; a.ldx = ldx; a.x_stride_g = 0;
   a.a_stride_g = 0; a.a_scale_stride_g = 0; a.b_stride_g = 0; a.b_scale_stride_g = 0;
   a.tiles_m = (int32_t)cdiv(M, 128); a.tiles_n = (int32_t)cdiv(N, 128);
-  a.offs = nullptr; a.num_groups = 0; a.row_index = nullptr;
+  a.offs = nullptr; a.num_groups = 0; a.row_index = nullptr; a.x2 = nullptr; a.ldx2 = 0; a.half = 0;
   const int eb = dtype == PT_F32 ? 4 : 2;
   a.vec_in = (N % 8 == 0) && ((ldx * eb) % 16 == 0) && (((uintptr_t)x) % 16 == 0);
   a.vec_out = (N % 8 == 0);
@@ -428,4 +469,46 @@ extern "C" int pt_quant_blockwise_transpose_batched(const void* x, int dtype, in
   a.vec_out_t = a.vec_out_t && ((N * K) % 16 == 0);
   a.vec_out = a.vec_out && ((N * K) % 8 == 0);
   return launch_quant<A_BLOCK, B_BLOCK, BL_TRANSPOSED, BS_MB_N>(a, dtype, G, (hipStream_t)stream);
+}
+
+// ---- SwiGLU fused into the activation quantisation --------------------------------------------
+template <int PRO>
+static int launch_silu_quant(const QuantArgs& a, hipStream_t stream) {
+  const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
+  if (blocks == 0) return PT_OK;
+  PT_REQUIRE(blocks < (1ll << 31), "quant: grid too large (%lld tiles)", (long long)blocks);
+  hipLaunchKernelGGL((pt::quant_tile_kernel<pt::bf16_tag, pt::A_ROW, pt::B_COL, pt::BL_TRANSPOSED, pt::BS_MB_N, PRO>),
+                     dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  return pt::check_launch("quant_tile_kernel(fused SwiGLU)");
+}
+
+extern "C" int pt_silu_mul_quant_rowwise_colwise(const void* gate_up, int64_t M, int64_t half, int64_t ld_gate_up,
+                                                 void* tok_fp8, float* tok_scale, void* ch_t_fp8, float* ch_scale,
+                                                 pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && half >= 0 && M % 128 == 0 && ld_gate_up >= 2 * half, "silu_mul_quant: bad shape");
+  if (M == 0 || half == 0) return PT_OK;
+  PT_REQUIRE(gate_up && tok_fp8 && tok_scale && ch_t_fp8 && ch_scale, "silu_mul_quant: null pointer");
+  PT_REQUIRE(half % 8 == 0 && ld_gate_up % 8 == 0 && ((uintptr_t)gate_up) % 16 == 0,
+             "silu_mul_quant: the half width and the row stride must be multiples of 8 elements, the pointer 16-byte aligned");
+  QuantArgs a;
+  fill_common(a, gate_up, PT_BF16, M, half, ld_gate_up);
+  a.half = half;
+  a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)ch_t_fp8; a.b_scale = ch_scale;
+  return launch_silu_quant<PRO_SILU_FWD>(a, (hipStream_t)stream);
+}
+
+extern "C" int pt_silu_mul_bwd_quant_rowwise_colwise(const void* grad_h, int64_t ld_grad_h, const void* gate_up,
+                                                     int64_t ld_gate_up, int64_t M, int64_t half, void* tok_fp8,
+                                                     float* tok_scale, void* ch_t_fp8, float* ch_scale, pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && half >= 0 && M % 128 == 0 && ld_gate_up >= 2 * half && ld_grad_h >= half, "silu_mul_bwd_quant: bad shape");
+  if (M == 0 || half == 0) return PT_OK;
+  PT_REQUIRE(grad_h && gate_up && tok_fp8 && tok_scale && ch_t_fp8 && ch_scale, "silu_mul_bwd_quant: null pointer");
+  PT_REQUIRE(half % 8 == 0 && ld_gate_up % 8 == 0 && ld_grad_h % 8 == 0 && ((uintptr_t)gate_up) % 16 == 0 &&
+                 ((uintptr_t)grad_h) % 16 == 0,
+             "silu_mul_bwd_quant: widths and row strides must be multiples of 8 elements, pointers 16-byte aligned");
+  QuantArgs a;
+  fill_common(a, grad_h, PT_BF16, M, 2 * half, ld_grad_h);
+  a.half = half; a.x2 = gate_up; a.ldx2 = ld_gate_up;
+  a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)ch_t_fp8; a.b_scale = ch_scale;
+  return launch_silu_quant<PRO_SILU_BWD>(a, (hipStream_t)stream);
 }

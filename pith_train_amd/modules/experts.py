@@ -20,6 +20,7 @@ import torch
 import torch.nn as nn
 
 from ..dualpipe_utils import FP8WeightCacheControl
+from ..operators import fused_experts
 from ..operators.clamped_swiglu import clamped_swiglu
 from ..operators.deepgemm_quantize import fp8cast_blockwise_transpose_batched
 from ..operators.grouped_linear import FP8GroupedLinear, FP8GroupedLinearFunc, GroupedLinearFunc
@@ -83,8 +84,17 @@ class Qwen35MoeExperts(nn.Module):
         self.gate_up_proj = training.GroupedLinear(num_experts, hidden_size, 2 * moe_intermediate_size)
         self.down_proj = training.GroupedLinear(num_experts, moe_intermediate_size, hidden_size)
 
-    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None):
-        """``row_map``: see :meth:`Qwen3MoeExperts.forward`."""
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None, fuse_activation: bool = True):
+        """``row_map``: see :meth:`Qwen3MoeExperts.forward`.  With ``fuse_activation`` (FP8 layers)
+        the block runs as one autograd node whose SwiGLU output and SwiGLU gradient are computed
+        inside the kernels that quantise them (same bits as the three-operator composition)."""
+        if (fuse_activation and training.fp8 and x.shape[0] > 0 and isinstance(self.gate_up_proj, FP8GroupedLinear)
+                and isinstance(self.down_proj, FP8GroupedLinear)
+                and fused_experts.supported(x, self.gate_up_proj.weight, self.down_proj.weight)):
+            return fused_experts.FP8SwiGLUExpertsFunc.apply(
+                x, self.gate_up_proj.weight, self.down_proj.weight, grouped_mm_offs, ks, ks_tensor,
+                self.gate_up_proj._get_quantized_weight(), self.down_proj._get_quantized_weight(), row_map,
+            )  # fmt: skip
         gi = precompute_group_indices(grouped_mm_offs, x.shape[0])
         kwargs = dict(grouped_mm_offs=grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, group_indices=gi)
         if row_map is not None:

@@ -1,0 +1,114 @@
+"""A whole SwiGLU expert block (fused gate_up projection -> SwiGLU -> down projection) as one
+autograd node, for the FP8 path.
+
+Composition and arithmetic are those of ``Qwen35MoeExperts.forward``
+(models/qwen35_moe.py:190-200) built from ``FP8GroupedLinearFunc`` (grouped_linear.py:104-236) and
+``silu_mul`` (silu_mul.py:93-143); the results are bit-identical to that composition.  Being one
+node lets two intermediate bf16 tensors stay out of memory: the SwiGLU output ``h`` (forward) and
+its gradient ``[dgate | dup]`` (backward) are produced inside the kernels that quantise them.
+The token permutation can be folded in as well (``row_map``, see ``FP8GroupedLinearFunc``).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+from .deepgemm_quantize import FP8, fp8cast_rowwise_colwise_t, fp8cast_rowwise_colwise_t_rows
+from .grouped_linear import m_grouped_fp8_gemm_nt, schedule_wgrad
+
+
+def _cdiv(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def silu_mul_quant(gate_up: torch.Tensor):
+    """``fp8cast_rowwise_colwise_t(silu_mul(gate_up[:, :I], gate_up[:, I:]))`` in one pass."""
+    M, two_i = gate_up.shape
+    half = two_i // 2
+    dev = gate_up.device
+    tok = torch.empty((M, half), dtype=FP8, device=dev)
+    tok_s = torch.empty((M, _cdiv(half, 128)), dtype=torch.float32, device=dev)
+    ch_t = torch.empty((half, M), dtype=FP8, device=dev)
+    ch_s = torch.empty((M // 128, half), dtype=torch.float32, device=dev)
+    _lib.call(
+        "pt_silu_mul_quant_rowwise_colwise", gate_up.data_ptr(), M, half, gate_up.stride(0),
+        tok.data_ptr(), tok_s.data_ptr(), ch_t.data_ptr(), ch_s.data_ptr(), _lib.stream_ptr(dev),
+    )  # fmt: skip
+    return tok, tok_s, ch_t, ch_s
+
+
+def silu_mul_bwd_quant(grad_h: torch.Tensor, gate_up: torch.Tensor):
+    """``fp8cast_rowwise_colwise_t`` of the SwiGLU gradient ``[dgate | dup]`` in one pass."""
+    M, two_i = gate_up.shape
+    half = two_i // 2
+    dev = gate_up.device
+    tok = torch.empty((M, two_i), dtype=FP8, device=dev)
+    tok_s = torch.empty((M, _cdiv(two_i, 128)), dtype=torch.float32, device=dev)
+    ch_t = torch.empty((two_i, M), dtype=FP8, device=dev)
+    ch_s = torch.empty((M // 128, two_i), dtype=torch.float32, device=dev)
+    _lib.call(
+        "pt_silu_mul_bwd_quant_rowwise_colwise", grad_h.data_ptr(), grad_h.stride(0), gate_up.data_ptr(),
+        gate_up.stride(0), M, half, tok.data_ptr(), tok_s.data_ptr(), ch_t.data_ptr(), ch_s.data_ptr(),
+        _lib.stream_ptr(dev),
+    )  # fmt: skip
+    return tok, tok_s, ch_t, ch_s
+
+
+def supported(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> bool:
+    """bf16 activations, half width and hidden size multiples of 8 (16-byte accesses)."""
+    half = w_gate_up.shape[1] // 2
+    return (x.dtype == torch.bfloat16 and w_gate_up.shape[1] % 2 == 0 and half % 8 == 0
+            and w_down.shape[1] % 8 == 0 and w_down.shape[2] == half)
+
+
+class FP8SwiGLUExpertsFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, w_gate_up, w_down, grouped_mm_offs, ks, ks_tensor, q_gate_up, q_down, row_map=None):
+        """``x`` is ``[M, K]`` grouped rows, or with ``row_map`` (int32 ``[M]``) the un-permuted
+        ``[m, K]`` tokens; the result has the same row layout as ``x``."""
+        _lib.require_cuda(x)
+        gu_fp8, gu_scale, gu_t_fp8, gu_t_scale = q_gate_up
+        dn_fp8, dn_scale, dn_t_fp8, dn_t_scale = q_down
+        num_groups, two_i, K = w_gate_up.shape
+        H = w_down.shape[1]
+        if row_map is not None:
+            M = row_map.shape[0]
+            x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, row_map)
+        else:
+            M = x.shape[0]
+            x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t(x)
+        gate_up = torch.empty((M, two_i), device=x.device, dtype=x.dtype)
+        m_grouped_fp8_gemm_nt((x_fp8, x_s), (gu_fp8, gu_scale), gate_up, grouped_mm_offs)
+        del x_fp8, x_s
+        h_fp8, h_s, h_ch_t, h_ch_s = silu_mul_quant(gate_up)
+        out = torch.empty((x.shape[0], H), device=x.device, dtype=x.dtype)
+        m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, row_map)
+        ctx.save_for_backward(gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, grouped_mm_offs, x_ch_t, x_ch_s,
+                              gate_up, h_ch_t, h_ch_s, row_map)
+        ctx.w_gate_up, ctx.w_down = w_gate_up, w_down
+        ctx.rows = (M, x.shape[0])
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, offs, x_ch_t, x_ch_s, gate_up, h_ch_t, h_ch_s,
+         row_map) = ctx.saved_tensors  # fmt: skip
+        w_gate_up, w_down = ctx.w_gate_up, ctx.w_down
+        M, rows_x = ctx.rows
+        half = gate_up.shape[1] // 2
+        K = w_gate_up.shape[2]
+        grad_out = grad_out.contiguous()
+        if row_map is not None:
+            dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t_rows(grad_out, row_map)
+        else:
+            dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t(grad_out)
+        grad_h = torch.empty((M, half), device=grad_out.device, dtype=grad_out.dtype)
+        m_grouped_fp8_gemm_nt((dy_fp8, dy_s), (dn_t_fp8, dn_t_scale), grad_h, offs)
+        schedule_wgrad(w_down, (dy_ch_t, dy_ch_s), (h_ch_t, h_ch_s), offs)
+        del dy_fp8, dy_s
+        dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s = silu_mul_bwd_quant(grad_h, gate_up)
+        grad_x = torch.empty((rows_x, K), device=grad_out.device, dtype=grad_out.dtype)
+        m_grouped_fp8_gemm_nt((dgu_fp8, dgu_s), (gu_t_fp8, gu_t_scale), grad_x, offs, row_map)
+        schedule_wgrad(w_gate_up, (dgu_ch_t, dgu_ch_s), (x_ch_t, x_ch_s), offs)
+        return grad_x, None, None, None, None, None, None, None, None

@@ -143,6 +143,39 @@ def k_grouped_fp8_wgrad(dy_t, x_t, out: torch.Tensor, grouped_mm_offs, accumulat
     return out
 
 
+def schedule_wgrad(weight: torch.Tensor, a_wgrad: tuple, b_wgrad: tuple, offs: torch.Tensor) -> None:
+    """Run - or, when ``WeightGradStore`` is enabled, queue - the weight-gradient GEMM of one
+    grouped linear (``grad_weight_fn``, grouped_linear.py:202-234): ``a_wgrad`` / ``b_wgrad`` are the
+    colwise-quantised transposed copies (fp8 ``[N, M]`` / ``[K, M]`` and their scales).  The result is
+    written to ``weight.grad`` (assigned if None, accumulated otherwise)."""
+    num_groups, N, K = weight.shape
+
+    def grad_weight_fn(a, b, offs):
+        # bf16(sum) is formed in the GEMM epilogue; an existing grad is accumulated there too
+        if weight.grad is None:
+            wg = torch.empty((num_groups, N, K), device=a[0].device, dtype=torch.bfloat16)
+            k_grouped_fp8_wgrad(a, b, wg, offs, accumulate=False)
+            weight.grad = wg if weight.dtype == torch.bfloat16 else wg.to(weight.dtype)
+        elif weight.grad.dtype == torch.bfloat16 and weight.grad.is_contiguous():
+            k_grouped_fp8_wgrad(a, b, weight.grad, offs, accumulate=True)
+        else:
+            wg = torch.empty((num_groups, N, K), device=a[0].device, dtype=torch.bfloat16)
+            k_grouped_fp8_wgrad(a, b, wg, offs, accumulate=False)
+            weight.grad += wg
+
+    if WeightGradStore.enabled:
+        WeightGradStore.put(
+            partial(
+                grad_weight_fn,
+                (a_wgrad[0].detach(), a_wgrad[1].detach()),
+                (b_wgrad[0].detach(), b_wgrad[1].detach()),
+                offs.detach(),
+            )
+        )
+    else:
+        grad_weight_fn(a_wgrad, b_wgrad, offs)
+
+
 class FP8GroupedLinearFunc(torch.autograd.Function):
     """FP8 grouped linear (grouped_linear.py:104-236): forward and dgrad are m-grouped NT GEMMs on
     1x128-scaled activations against 128x128-scaled weights, wgrad a k-grouped GEMM on the colwise
@@ -211,32 +244,7 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
             (grad_fp8, scale_grad), (weight_t_fp8, scale_weight_t), grad_input, offs, in_rows
         )
 
-        def grad_weight_fn(a, b, offs):
-            # bf16(sum) is formed in the GEMM epilogue; an existing grad is accumulated there too
-            if weight.grad is None:
-                wg = torch.empty((num_groups, N, K), device=a[0].device, dtype=torch.bfloat16)
-                k_grouped_fp8_wgrad(a, b, wg, offs, accumulate=False)
-                weight.grad = wg if weight.dtype == torch.bfloat16 else wg.to(weight.dtype)
-            elif weight.grad.dtype == torch.bfloat16 and weight.grad.is_contiguous():
-                k_grouped_fp8_wgrad(a, b, weight.grad, offs, accumulate=True)
-            else:
-                wg = torch.empty((num_groups, N, K), device=a[0].device, dtype=torch.bfloat16)
-                k_grouped_fp8_wgrad(a, b, wg, offs, accumulate=False)
-                weight.grad += wg
-
-        a_wgrad = (grad_ch_t, scale_grad_ch)
-        b_wgrad = (input_ch_t, scale_input_ch)
-        if WeightGradStore.enabled:
-            WeightGradStore.put(
-                partial(
-                    grad_weight_fn,
-                    (a_wgrad[0].detach(), a_wgrad[1].detach()),
-                    (b_wgrad[0].detach(), b_wgrad[1].detach()),
-                    offs.detach(),
-                )
-            )
-        else:
-            grad_weight_fn(a_wgrad, b_wgrad, offs)
+        schedule_wgrad(weight, (grad_ch_t, scale_grad_ch), (input_ch_t, scale_input_ch), offs)
         return grad_input, None, None, None, None, None, None, None, None, None
 
 

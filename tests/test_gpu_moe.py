@@ -108,18 +108,25 @@ def test_stage3_permute_folded_into_quant_and_gemm_is_bit_identical(kind, E, H, 
     tokens = torch.randn((T * k, H), generator=g).bfloat16().cuda()
     dy = torch.randn((T * k, H), generator=g).bfloat16().cuda()
     w = _weights(kind, E, H, I, 5)
+    import functools
+
     res = []
-    for fuse in (True, False):
+    for fuse, fuse_act in ((True, True), (False, False), (False, True), (True, False)):
         mod, params = _build(kind, E, H, I, w)
+        if kind == "fused":  # the one-node SwiGLU block exists for the fused gate_up layout
+            mod.forward = functools.partial(mod.forward, fuse_activation=fuse_act)
+        elif fuse_act != fuse:
+            continue
         FP8WeightCacheControl.step()
         tok = tokens.clone().requires_grad_(True)
         out = forward_stage3(mod, tok, ids.reshape(-1).cuda(), E, fuse_permute=fuse)
         out.backward(dy)
         res.append((out.detach(), tok.grad, {n: p.grad for n, p in params.items()}))
-    assert torch.equal(res[0][0], res[1][0]), "forward output differs"
-    assert torch.equal(res[0][1], res[1][1]), "token gradient differs"
-    for n in res[0][2]:
-        assert torch.equal(res[0][2][n], res[1][2][n]), f"{n} gradient differs"
+    for other in res[1:]:
+        assert torch.equal(res[0][0], other[0]), "forward output differs"
+        assert torch.equal(res[0][1], other[1]), "token gradient differs"
+        for n in res[0][2]:
+            assert torch.equal(res[0][2][n], other[2][n]), f"{n} gradient differs"
 
 
 def test_stage3_with_dedup_expand_fused_and_unfused():
