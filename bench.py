@@ -162,8 +162,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="qwen3-30b-a3b-moe", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cached-weights", action="store_true",
-                    help="also report a step time with the FP8 weight cache kept across steps")
+    ap.add_argument("--no-cached-weights", action="store_true",
+                    help="skip the extra (untimed-for-value) pass that keeps the FP8 weight cache across steps")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region launch gather_rows_kernel as a plain copy of 256 MiB "
                          "(identity index) three times: the known-size kernel that FETCH_SIZE / "
@@ -223,7 +223,9 @@ def main():
     achieved = flops * args.steps / (gemm_ms * 1e-3) / 1e12 if gemm_ms > 0 else 0.0
 
     extra = {}
-    if args.cached_weights:
+    if not args.no_cached_weights:
+        # secondary figure: the reference quantises weights once per optimizer step and reuses them
+        # for every micro-batch; `value` above re-quantises them in every step
         for _ in range(2):
             step(bump=False)
         torch.cuda.synchronize()
@@ -231,7 +233,10 @@ def main():
         for _ in range(args.steps):
             step(bump=False)
         torch.cuda.synchronize()
-        extra["ms_per_step_weights_cached"] = (time.perf_counter() - t1) / args.steps * 1e3
+        ms_c = (time.perf_counter() - t1) / args.steps * 1e3
+        extra["weights_cached"] = {"ms_per_step": ms_c, "value": flops / (ms_c * 1e-3) / 1e12, "unit": "TFLOP/s",
+                                   "note": "FP8 weight cache kept across steps (one quantisation per optimizer step, "
+                                           "as FP8WeightCacheControl does); not the headline value"}
 
     if args.calibrate_copy:
         cr, ch = 65536, 2048  # 65536 rows x 2048 bf16 = 256 MiB read + 256 MiB written (+ 512 KiB of indices)
@@ -260,7 +265,8 @@ def main():
         "data": "synthetic (seed 0: x~N(0,1) bf16, weights~N(0,0.02), grad~N(0,1), router logits~N(0,1) softmax top-k)",
         "config": {
             "workload": args.workload, "kind": kind, "hidden": H, "moe_intermediate": I, "experts": E,
-            "top_k": k, "tokens": T, "routed_rows": rows, "algorithmic_gemm_tflop_per_step": flops / 1e12,
+            "top_k": k, "tokens": T, "routed_rows": rows, "zipf_s": zipf,
+            "algorithmic_gemm_tflop_per_step": flops / 1e12,
             "weight_quant_in_step": True,
         },
         "roofline": {

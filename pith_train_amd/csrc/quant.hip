@@ -158,10 +158,23 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
     }
   } else if (p.vec_in) {
     const bool col_ok = col0 < p.N;
+    int32_t src[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) src[i] = 0;
+    if (p.row_index) {
+      if (row0 + 8 <= p.M) {  // the thread's 8 rows are consecutive: two 16-byte index loads (row0 % 8 == 0)
+        const int4 lo = *reinterpret_cast<const int4*>(p.row_index + row0);
+        const int4 hi = *reinterpret_cast<const int4*>(p.row_index + row0 + 4);
+        src[0] = lo.x; src[1] = lo.y; src[2] = lo.z; src[3] = lo.w; src[4] = hi.x; src[5] = hi.y; src[6] = hi.z; src[7] = hi.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (row0 + i < p.M) src[i] = p.row_index[row0 + i];
+      }
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      int64_t sr = row0 + i;
-      if (p.row_index && sr < p.M) sr = p.row_index[sr];
+      const int64_t sr = p.row_index ? (int64_t)src[i] : row0 + i;
       if (col_ok && row0 + i < p.M && sr >= 0) f.load_row(i, xb + (sr * p.ldx + col0) * Loader<T>::kBytes);
       else f.zero_row(i);
     }
@@ -190,6 +203,43 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) rowmax[i] = row16_allmax(rowmax[i]);
   }
+
+  auto write_same_orientation = [&](float blk_scale, float blk_rcp) {
+  f.fence();
+  {
+    uint8_t* ab = p.a_out + g * p.a_stride_g;
+    const int64_t nb = p.tiles_n;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      f.fence_row(i);
+      float rcp;
+      if (AM == A_ROW) {
+        const float s = fp8_scale_from_amax(rowmax[i], rcp);
+        if (cc == 0 && row0 + i < p.M) p.a_scale[(row0 + i) * nb + tc] = s;
+      } else {
+        rcp = blk_rcp;
+      }
+      const uint32_t lo = cvt4_e4m3(f.get(i, 0) * rcp, f.get(i, 1) * rcp, f.get(i, 2) * rcp, f.get(i, 3) * rcp);
+      const uint32_t hi = cvt4_e4m3(f.get(i, 4) * rcp, f.get(i, 5) * rcp, f.get(i, 6) * rcp, f.get(i, 7) * rcp);
+      if (row0 + i < p.M) {
+        uint8_t* dst = ab + (row0 + i) * p.N + col0;
+        if (p.vec_out) {
+          if (col0 < p.N) *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (col0 + j < p.N) dst[j] = (uint8_t)(((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xFF);
+        }
+      }
+    }
+    if (AM == A_BLOCK && t == 0)
+      p.a_scale[g * p.a_scale_stride_g + (int64_t)tr * p.tiles_n + tc] = blk_scale;
+  }
+
+  };
+  // Row-scaled output needs nothing from the other phases: write it now so that the row maxima
+  // are dead before the column phase starts (fewer live registers, more resident waves).
+  if (AM == A_ROW) write_same_orientation(0.f, 0.f);
 
   f.fence();
   float colmax[8];
@@ -231,37 +281,8 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
     blk_scale = fp8_scale_from_amax(blkmax, blk_rcp);
   }
 
-  // ---- same-orientation output -----------------------------------------------------------
-  f.fence();
-  {
-    uint8_t* ab = p.a_out + g * p.a_stride_g;
-    const int64_t nb = p.tiles_n;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      f.fence_row(i);
-      float rcp;
-      if (AM == A_ROW) {
-        const float s = fp8_scale_from_amax(rowmax[i], rcp);
-        if (cc == 0 && row0 + i < p.M) p.a_scale[(row0 + i) * nb + tc] = s;
-      } else {
-        rcp = blk_rcp;
-      }
-      const uint32_t lo = cvt4_e4m3(f.get(i, 0) * rcp, f.get(i, 1) * rcp, f.get(i, 2) * rcp, f.get(i, 3) * rcp);
-      const uint32_t hi = cvt4_e4m3(f.get(i, 4) * rcp, f.get(i, 5) * rcp, f.get(i, 6) * rcp, f.get(i, 7) * rcp);
-      if (row0 + i < p.M) {
-        uint8_t* dst = ab + (row0 + i) * p.N + col0;
-        if (p.vec_out) {
-          if (col0 < p.N) *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
-        } else {
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            if (col0 + j < p.N) dst[j] = (uint8_t)(((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xFF);
-        }
-      }
-    }
-    if (AM == A_BLOCK && t == 0)
-      p.a_scale[g * p.a_scale_stride_g + (int64_t)tr * p.tiles_n + tc] = blk_scale;
-  }
+  // ---- same-orientation output (row-scaled: already written above) ---------------------------
+  if (AM != A_ROW) write_same_orientation(blk_scale, blk_rcp);
 
   // ---- twin ---------------------------------------------------------------------------------
   f.fence();
