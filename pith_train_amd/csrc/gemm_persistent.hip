@@ -109,13 +109,14 @@ __device__ __forceinline__ void store_staged_bf16(const v16f& a, __amdgpu_buffer
                                                   uint32_t soff, uint32_t pitch, bool accumulate, int lane) {
   const bool odd = lane & 1;
   uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 64 + ((lane & 31) >> 1) * 4;
+  // p = (row r | row r+1) of the lane's column; the even lane of a pair takes both low halves (row r,
+  // columns c and c+1), the odd lane both high halves (row r+1): one byte permute of own and neighbour
+  const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
 #pragma unroll
   for (int v = 0; v < 16; v += 2) {
-    const float x0 = a[v], x1 = a[v + 1];
-    const float send = odd ? x0 : x1;
-    const float recv = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send), 0xB1, 0xF, 0xF, false));
-    const uint32_t w = odd ? pack2_bf16(recv, x1) : pack2_bf16(x0, recv);
-    *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = w;
+    const uint32_t pk = pack2_bf16(a[v], a[v + 1]);
+    const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, false);
+    *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = __builtin_amdgcn_perm(nb, pk, sel);
   }
   // the reads below alias the writes above: keep the compiler from reordering them and let the
   // writes land first
@@ -144,13 +145,14 @@ __device__ __forceinline__ void store_staged_bf16_rows(const v16f& a, __amdgpu_b
                                                        uint32_t voff1, uint32_t soff, int lane) {
   const bool odd = lane & 1;
   uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 64 + ((lane & 31) >> 1) * 4;
+  // p = (row r | row r+1) of the lane's column; the even lane of a pair takes both low halves (row r,
+  // columns c and c+1), the odd lane both high halves (row r+1): one byte permute of own and neighbour
+  const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
 #pragma unroll
   for (int v = 0; v < 16; v += 2) {
-    const float x0 = a[v], x1 = a[v + 1];
-    const float send = odd ? x0 : x1;
-    const float recv = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send), 0xB1, 0xF, 0xF, false));
-    const uint32_t w = odd ? pack2_bf16(recv, x1) : pack2_bf16(x0, recv);
-    *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = w;
+    const uint32_t pk = pack2_bf16(a[v], a[v + 1]);
+    const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, false);
+    *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = __builtin_amdgcn_perm(nb, pk, sel);
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   const uint8_t* rd = stg + (lane >> 2) * 64 + (lane & 3) * 16;
@@ -245,7 +247,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   const int t_step = gridDim.x >> 3;
   const int t_first = xcd * per_xcd + (blockIdx.x >> 3);
 
-  auto decode = [&](int t, Tile& T) {
+  auto decode = [&](int t, Tile& T, int& hint) {
     if (MODE == GEMM_DENSE) {
       T.g = 0;
       // The 32 CUs of an XCD work on 32 consecutive logical tiles at a time; laying those out as
@@ -268,12 +270,11 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
       T.a_lim = (int)p.rows_a; T.b_lim = (int)p.rows_b; T.k_begin = 0; T.k_len = (int)p.red; T.kb0 = 0;
     } else if (MODE == GEMM_M_GROUPED) {
       const int q = t / p.tiles_b;
-      int lo = 1, hi = p.G;  // first j in [1, G] with s_pref[j] > q
-      while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (s_pref[mid] > q) hi = mid; else lo = mid + 1;
-      }
-      const int g = __builtin_amdgcn_readfirstlane(lo - 1);
+      // a cursor visits tiles in increasing order: walk on from the group of its previous tile
+      int gg = hint;
+      while (gg + 1 < p.G && __builtin_amdgcn_readfirstlane(s_pref[gg + 1]) <= q) ++gg;
+      hint = gg;
+      const int g = gg;
       const int pg = __builtin_amdgcn_readfirstlane(s_pref[g]), pg1 = __builtin_amdgcn_readfirstlane(s_pref[g + 1]);
       const int gs = g ? p.offs[g - 1] : 0;
       const int m_tiles = pg1 - pg;
@@ -321,13 +322,14 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   // ---- loader: walks (tile, 128-block) pairs ahead of the MFMAs and keeps the LDS ring full ----
   Tile L;
   int lt = t_first - t_step, l_it = 0, l_nk = 0, n_issued = 0;
+  int l_hint = 0, p_hint = 0, c_hint = 0;  // per-cursor group of the last decoded tile (m-grouped mode)
   v4i rs_b = rs_a, rs_sb = rs_sa;
   uint32_t vs[SPW];  // this wave's per-lane scale offsets (bytes) at step 0 of the loader's tile
   auto issue_stage = [&]() {
     while (l_it >= l_nk) {
       lt += t_step;
       if (lt >= t_end) return;
-      decode(lt, L);
+      decode(lt, L, l_hint);
       l_it = 0;
       l_nk = (L.k_len + 127) >> 7;
       rs_b = make_rsrc(p.b + (MODE == GEMM_M_GROUPED ? (int64_t)L.g * p.b_stride_g : 0), (uint32_t)p.b_bytes);
@@ -389,7 +391,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
     while (p_it >= p_nk) {
       pt += t_step;
       if (pt >= t_end) return;
-      decode(pt, Pf);
+      decode(pt, Pf, p_hint);
       p_it = 0;
       p_nk = (Pf.k_len + 127) >> 7;
       rs_b_pf = make_rsrc(p.b + (MODE == GEMM_M_GROUPED ? (int64_t)Pf.g * p.b_stride_g : 0), (uint32_t)p.b_bytes);
@@ -437,7 +439,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   Tile C;
 #pragma unroll 1
   for (int t = t_first; t < t_end; t += t_step) {
-    decode(t, C);
+    decode(t, C, c_hint);
     const int nk = (C.k_len + 127) >> 7;
     // Waves whose whole row range lies past the end of a ragged group skip the MFMAs (they still
     // take part in the loads and barriers).
