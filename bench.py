@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 # Average HBM bytes moved by one GEMM launch (fetch + write), from the FETCH_SIZE / WRITE_SIZE
 # counter runs summarised under profiles/ (scaled by the same counters' readings for a plain copy
 # of known size).  None for a workload that has no counter run.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-30b-a3b-moe": 855e6}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-30b-a3b-moe": 800e6}
 
 WORKLOADS = {
     # name: (kind, hidden, intermediate, experts, top_k, tokens, zipf)
@@ -121,6 +121,68 @@ class GemmTimer:
         return {k: {"ms_total": v[0], "launches": v[1]} for k, v in out.items()}
 
 
+def hbm_kernel_report(H, I, E, rows, eidx):
+    """HIP-event timings of the HBM-bound kernels of the path at this workload's shapes, called
+    through the operator layer one at a time: achieved GB/s = algorithmic bytes (2 B per bf16,
+    1 B per fp8 element, 4 B per 128-element scale) / time, against the 8 TB/s HBM peak."""
+    import torch
+
+    from pith_train_amd.operators import deepgemm_quantize as Q
+    from pith_train_amd.operators import fused_experts as FE
+    from pith_train_amd.operators import token_scatter as TS
+    from pith_train_amd.operators.silu_mul import silu_mul_halves
+
+    def timeit(fn, iters=10):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(iters):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / iters * 1e3  # us
+
+    out = []
+
+    def rep(name, us, nbytes):
+        gbs = nbytes / us / 1e3
+        out.append({"kernel": name, "us": round(us, 1), "algorithmic_MB": round(nbytes / 1e6, 1),
+                    "GB/s": round(gbs, 0), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 3)})
+
+    g = torch.Generator(device="cuda").manual_seed(0)
+    src = torch.randn((rows, H), device="cuda", generator=g).bfloat16()
+    xp, reverse, offs, ks, ks_tensor = TS.scatter_for_grouped_gemm(src, eidx, E)
+    Mp = xp.shape[0]
+    _, _, _, _, src_of = TS.group_rows_with_sizes(eidx, E)
+    sc = 4.0 / 128
+    rep("quant_tile_kernel rowwise+colwise [Mp,H]", timeit(lambda: Q.fp8cast_rowwise_colwise_t(xp)), Mp * H * (4 + 2 * sc))
+    rep("quant_tile_kernel rowwise+colwise of gathered rows [Mp,H]",
+        timeit(lambda: Q.fp8cast_rowwise_colwise_t_rows(src, src_of)), (rows * 2 + Mp * (2 + 2 * sc)) * H + 4 * Mp)
+    w = (torch.randn((E, 2 * I, H), device="cuda", generator=g) * 0.02).bfloat16()
+    rep("quant_tile_kernel 128x128 blockwise + transpose [E,2I,H]",
+        timeit(lambda: Q.fp8cast_blockwise_transpose_batched(w)), w.numel() * 4.0)
+    del w
+    gu = torch.randn((Mp, 2 * I), device="cuda", generator=g).bfloat16()
+    dh = torch.randn((Mp, I), device="cuda", generator=g).bfloat16()
+    rep("quant_tile_kernel SwiGLU fwd + quant [Mp,I]", timeit(lambda: FE.silu_mul_quant(gu)), Mp * I * (4 + 2 + 2 * sc))
+    rep("quant_tile_kernel SwiGLU bwd + quant [Mp,2I]", timeit(lambda: FE.silu_mul_bwd_quant(dh, gu)),
+        Mp * I * (2 + 4 + 2 * (2 + 2 * sc)))
+    gur = gu.clone().requires_grad_(True)
+    rep("silu_mul_2d_kernel fwd [Mp,I]", timeit(lambda: silu_mul_halves(gur)), Mp * I * 6)
+    o = silu_mul_halves(gur)
+    rep("silu_mul_2d_kernel bwd [Mp,I]", timeit(lambda: torch.autograd.grad(o, gur, dh, retain_graph=True)), Mp * I * 10)
+    del gu, dh, gur, o
+    rep("group_rows + permute_rows_kernel (scatter_for_grouped_gemm) [rows,H]",
+        timeit(lambda: TS.scatter_for_grouped_gemm(src, eidx, E)), (rows + Mp) * H * 2 + 16 * rows)
+    rep("gather_rows_kernel (padded_index_gather) [rows,H]", timeit(lambda: TS.padded_index_gather(xp, reverse)),
+        2 * rows * H * 2 + 8 * rows)
+    rep("gb_* kernels (padded_index_gather backward) [rows,H]",
+        timeit(lambda: TS._PaddedIndexGather.scatter_sum(src, reverse, Mp, 1024)), (rows + Mp) * H * 2 + 12 * rows)
+    return out
+
+
 def cpu_baseline(kind, H, I, E, k, T, zipf, budget_s=12.0):
     """The CPU oracle of the same layer on the same seeded inputs: the BF16 grouped-linear
     semantics (the reference's pure-PyTorch path), forward + backward, all host cores given to
@@ -164,6 +226,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cached-weights", action="store_true",
                     help="skip the extra (untimed-for-value) pass that keeps the FP8 weight cache across steps")
+    ap.add_argument("--no-kernel-report", action="store_true",
+                    help="skip the per-kernel GB/s table of the HBM-bound kernels (hbm_kernels in the JSON line)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region launch gather_rows_kernel as a plain copy of 256 MiB "
                          "(identity index) three times: the known-size kernel that FETCH_SIZE / "
@@ -285,6 +349,8 @@ def main():
         },
         **extra,
     }
+    if not args.no_kernel_report:
+        result["hbm_kernels"] = hbm_kernel_report(H, I, E, rows, eidx)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(kind, H, I, E, k, T, zipf)
     print(json.dumps(result))
