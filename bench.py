@@ -38,7 +38,39 @@ WORKLOADS = {
     "toy": ("split", 256, 512, 8, 2, 1024, None),
     "dsv2-lite-moe": ("split", 2048, 1408, 64, 6, 8192, 1.2),
     "gpt-oss-20b-moe": ("gpt_oss", 2880, 2880, 32, 4, 16384, None),
+    "qwen3-decoder-linears-32k": ("fused", 2048, 768, 128, 8, 32768, None),
 }
+# Parts of a workload beyond the routed experts (all on the same tokens):
+#   shared_mlp: width of a dense FP8 SwiGLU MLP (DeepSeek-V2-Lite's two shared experts run as one);
+#   dense_linears: (in, out) of dense FP8 linears (q, k, v, o projections of the decoder layer);
+#   dedup_fraction: share of routed rows that re-use an already received token row (the rows reach the
+#   experts through the dedup expand index instead of being materialised).
+EXTRAS = {
+    "dsv2-lite-moe": {"shared_mlp": 2816},
+    "qwen3-decoder-linears-32k": {"dense_linears": [(2048, 4096), (2048, 512), (2048, 512), (4096, 2048)],
+                                  "dedup_fraction": 0.25},
+}
+
+
+def extra_flops(extras, T, H):
+    """Algorithmic GEMM FLOPs (fwd + dgrad + wgrad) of the dense parts."""
+    f = 0.0
+    if "shared_mlp" in extras:
+        f += 3 * 6.0 * T * H * extras["shared_mlp"]
+    for fin, fout in extras.get("dense_linears", []):
+        f += 3 * 2.0 * T * fin * fout
+    return f
+
+
+def make_dedup_expand(rows, fraction, seed=0):
+    """expand_idx[rows] into U = rows * (1 - fraction) unique received rows: every unique row is
+    referenced at least once, the remaining references are uniform repeats."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed + 1)
+    U = int(round(rows * (1.0 - fraction)))
+    idx = torch.cat([torch.arange(U), torch.randint(0, U, (rows - U,), generator=g)])
+    return idx[torch.randperm(rows, generator=g)], U
 
 
 def make_inputs(kind, H, I, E, k, T, zipf, seed=0):
@@ -247,14 +279,40 @@ def main():
 
     _lib.load()  # fail loudly if the HIP library is missing
     kind, H, I, E, k, T, zipf = WORKLOADS[args.workload]
+    extras = EXTRAS.get(args.workload, {})
     ids, x, dy, w = make_inputs(kind, H, I, E, k, T, zipf)
     mod = build_module(kind, H, I, E, w)
     params = [p for p in mod.parameters()]
-    tokens = x.cuda().unsqueeze(1).expand(-1, k, -1).reshape(-1, H).contiguous()
     eidx = ids.reshape(-1).cuda()
     dyc = dy.cuda()
     rows = T * k
-    flops = OM.gemm_flops(rows, H, I)
+    expand_idx = None
+    if "dedup_fraction" in extras:
+        # the experts receive only the unique rows and re-expand them through expand_idx
+        expand_cpu, U = make_dedup_expand(rows, extras["dedup_fraction"])
+        g = torch.Generator().manual_seed(2)
+        tokens = torch.randn((U, H), generator=g).bfloat16().cuda()
+        expand_idx = expand_cpu.cuda()
+    else:
+        tokens = x.cuda().unsqueeze(1).expand(-1, k, -1).reshape(-1, H).contiguous()
+    flops = OM.gemm_flops(rows, H, I) + extra_flops(extras, T, H)
+    dense = []  # (module, input [T, in], upstream grad [T, out])
+    if extras.get("shared_mlp") or extras.get("dense_linears"):
+        from pith_train_amd.modules import training
+        from pith_train_amd.modules.experts import DeepSeekV2MLP
+
+        g = torch.Generator().manual_seed(3)
+        mk = lambda *s_: torch.randn(s_, generator=g).bfloat16().cuda()  # noqa: E731
+        if extras.get("shared_mlp"):
+            m = DeepSeekV2MLP(H, extras["shared_mlp"]).cuda().to(torch.bfloat16)
+            dense.append((m, mk(T, H), mk(T, H)))
+        for fin, fout in extras.get("dense_linears", []):
+            m = training.Linear(fin, fout, bias=False).cuda().to(torch.bfloat16)
+            dense.append((m, mk(T, fin), mk(T, fout)))
+        with torch.no_grad():
+            for m, _, _ in dense:
+                for p_ in m.parameters():
+                    p_.copy_((torch.randn(p_.shape, generator=g) * 0.02).to(p_.dtype))
     timer = GemmTimer().install()
 
     def step(bump=True):
@@ -263,10 +321,13 @@ def main():
         for p in params:
             p.grad = None
         tok = tokens.detach().requires_grad_(True)
-        out = forward_stage3(mod, tok, eidx, E)
+        out = forward_stage3(mod, tok, eidx, E, expand_idx=expand_idx)
         # weight gradients are written to .grad by the wgrad GEMM itself; the token gradient is
         # taken directly (a leaf's .grad would cost a clone that no training step performs)
         (dtok,) = torch.autograd.grad(out, tok, dyc)
+        for m, xin, gout in dense:
+            xi = xin.detach().requires_grad_(True)
+            torch.autograd.grad(m(xi), [xi] + list(m.parameters()), gout)
         return dtok
 
     for _ in range(args.warmup):
@@ -329,7 +390,7 @@ def main():
         "data": "synthetic (seed 0: x~N(0,1) bf16, weights~N(0,0.02), grad~N(0,1), router logits~N(0,1) softmax top-k)",
         "config": {
             "workload": args.workload, "kind": kind, "hidden": H, "moe_intermediate": I, "experts": E,
-            "top_k": k, "tokens": T, "routed_rows": rows, "zipf_s": zipf,
+            "top_k": k, "tokens": T, "routed_rows": rows, "zipf_s": zipf, **extras,
             "algorithmic_gemm_tflop_per_step": flops / 1e12,
             "weight_quant_in_step": True,
         },
@@ -353,6 +414,8 @@ def main():
         result["hbm_kernels"] = hbm_kernel_report(H, I, E, rows, eidx)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(kind, H, I, E, k, T, zipf)
+        if extras:
+            result["cpu_baseline"]["sample"] += " (routed experts only; the dense parts of this workload are not in the CPU figure)"
     print(json.dumps(result))
 
 
