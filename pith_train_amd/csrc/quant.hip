@@ -99,7 +99,7 @@ template <> struct Frag<float> {
   __device__ __forceinline__ void fence_row(int) {}
 };
 
-enum { PRO_NONE = 0, PRO_SILU_FWD = 1, PRO_SILU_BWD = 2 };  // what the tile is computed from
+enum { PRO_NONE = 0, PRO_SILU_FWD = 1, PRO_SILU_BWD = 2, PRO_SILU_BWD_PAIR = 3 };  // what the tile is computed from
 
 template <typename T, int AM, int BMODE, int BL, int BS, int PRO = PRO_NONE>
 __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
@@ -110,7 +110,10 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   const int t = threadIdx.x;
   const int cc = t & 15, rg = t >> 4, wave = t >> 6, lane = t & 63;
   int64_t bid = blockIdx.x;
-  const int tc = (int)(bid % p.tiles_n); bid /= p.tiles_n;
+  // PRO_SILU_BWD_PAIR: one workgroup produces the dgate tile and its dup twin (half / 128 column
+  // tiles further right) from one read of grad_h, gate and up
+  const int tiles_n_grid = PRO == PRO_SILU_BWD_PAIR ? p.tiles_n / 2 : p.tiles_n;
+  const int tc = (int)(bid % tiles_n_grid); bid /= tiles_n_grid;
   const int tr = (int)(bid % p.tiles_m);
   const int64_t g = bid / p.tiles_m;
 
@@ -119,7 +122,30 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   const char* xb = reinterpret_cast<const char*>(p.x) + g * p.x_stride_g * Loader<T>::kBytes;
 
   Frag<T> f;
-  if constexpr (PRO != PRO_NONE) {
+  [[maybe_unused]] Frag<T> f_up;  // PRO_SILU_BWD_PAIR only
+  if constexpr (PRO == PRO_SILU_BWD_PAIR) {
+    const bool col_ok = col0 < p.half;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (col_ok && row0 + i < p.M) {
+        const int64_t r = row0 + i;
+        float d[8], g[8], u[8], dg[8], du[8];
+        st_bf16::load8(xb + (r * p.ldx + col0) * 2, d);
+        const char* gp = (const char*)p.x2 + (r * p.ldx2 + col0) * 2;
+        st_bf16::load8(gp, g);
+        st_bf16::load8(gp + p.half * 2, u);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) silu_mul_b(d[j], g[j], u[j], dg[j], du[j]);
+        f.w[i][0] = pack_bf16x2(dg[0], dg[1]); f.w[i][1] = pack_bf16x2(dg[2], dg[3]);
+        f.w[i][2] = pack_bf16x2(dg[4], dg[5]); f.w[i][3] = pack_bf16x2(dg[6], dg[7]);
+        f_up.w[i][0] = pack_bf16x2(du[0], du[1]); f_up.w[i][1] = pack_bf16x2(du[2], du[3]);
+        f_up.w[i][2] = pack_bf16x2(du[4], du[5]); f_up.w[i][3] = pack_bf16x2(du[6], du[7]);
+      } else {
+        f.zero_row(i);
+        f_up.zero_row(i);
+      }
+    }
+  } else if constexpr (PRO != PRO_NONE) {
     // The quantised tensor is the bf16-rounded SwiGLU output (forward: h = silu(gate) * up from
     // gate_up = x) or its gradient (backward: [dgate | dup] from grad_h = x and gate_up = x2),
     // computed here instead of being written to memory and read back.  bf16 only, 16-byte loads.
@@ -190,6 +216,8 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
     }
   }
 
+  // Everything after the load stage, for one 128x128 tile held in `f` at column tile `tc`.
+  auto quantise_tile = [&](const int tc, const int64_t col0, Frag<T>& f) {
   // ---- reductions ------------------------------------------------------------------------
   float rowmax[8];
 #pragma unroll
@@ -372,6 +400,12 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
       }
     }
   }
+  };
+  quantise_tile(tc, col0, f);
+  if constexpr (PRO == PRO_SILU_BWD_PAIR) {
+    __syncthreads();  // the shared staging arrays are reused by the twin
+    quantise_tile(tc + p.tiles_n / 2, col0 + p.half, f_up);
+  }
 }
 
 template <int AM, int BMODE, int BL, int BS>
@@ -495,7 +529,7 @@ extern "C" int pt_quant_blockwise_transpose_batched(const void* x, int dtype, in
 // ---- SwiGLU fused into the activation quantisation --------------------------------------------
 template <int PRO>
 static int launch_silu_quant(const QuantArgs& a, hipStream_t stream) {
-  const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n;
+  const int64_t blocks = (int64_t)a.tiles_m * (PRO == PRO_SILU_BWD_PAIR ? a.tiles_n / 2 : a.tiles_n);
   if (blocks == 0) return PT_OK;
   PT_REQUIRE(blocks < (1ll << 31), "quant: grid too large (%lld tiles)", (long long)blocks);
   hipLaunchKernelGGL((pt::quant_tile_kernel<pt::bf16_tag, pt::A_ROW, pt::B_COL, pt::BL_TRANSPOSED, pt::BS_MB_N, PRO>),
@@ -531,5 +565,7 @@ extern "C" int pt_silu_mul_bwd_quant_rowwise_colwise(const void* grad_h, int64_t
   fill_common(a, grad_h, PT_BF16, M, 2 * half, ld_grad_h);
   a.half = half; a.x2 = gate_up; a.ldx2 = ld_gate_up;
   a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)ch_t_fp8; a.b_scale = ch_scale;
+  // with whole 128-column tiles per half, each workgroup makes a dgate tile and its dup twin
+  if (half % 128 == 0) return launch_silu_quant<PRO_SILU_BWD_PAIR>(a, (hipStream_t)stream);
   return launch_silu_quant<PRO_SILU_BWD>(a, (hipStream_t)stream);
 }
