@@ -247,7 +247,9 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   const int t_step = gridDim.x >> 3;
   const int t_first = xcd * per_xcd + (blockIdx.x >> 3);
 
-  auto decode = [&](int t, Tile& T, int& hint) {
+  // geometry of logical tile t; plain per-lane arithmetic (used by every lane for a different t
+  // when the tile table is built, and uniformly beyond the table)
+  auto decode_any = [&](int t, Tile& T) {
     if (MODE == GEMM_DENSE) {
       T.g = 0;
       // The 32 CUs of an XCD work on 32 consecutive logical tiles at a time; laying those out as
@@ -270,12 +272,13 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
       T.a_lim = (int)p.rows_a; T.b_lim = (int)p.rows_b; T.k_begin = 0; T.k_len = (int)p.red; T.kb0 = 0;
     } else if (MODE == GEMM_M_GROUPED) {
       const int q = t / p.tiles_b;
-      // a cursor visits tiles in increasing order: walk on from the group of its previous tile
-      int gg = hint;
-      while (gg + 1 < p.G && __builtin_amdgcn_readfirstlane(s_pref[gg + 1]) <= q) ++gg;
-      hint = gg;
-      const int g = gg;
-      const int pg = __builtin_amdgcn_readfirstlane(s_pref[g]), pg1 = __builtin_amdgcn_readfirstlane(s_pref[g + 1]);
+      int lo = 1, hi = p.G;  // first j in [1, G] with s_pref[j] > q
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (s_pref[mid] > q) hi = mid; else lo = mid + 1;
+      }
+      const int g = lo - 1;
+      const int pg = s_pref[g], pg1 = s_pref[g + 1];
       const int gs = g ? p.offs[g - 1] : 0;
       const int m_tiles = pg1 - pg;
       const int idx = t - pg * p.tiles_b;
@@ -290,6 +293,40 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
       T.a_row0 = (idx % p.tiles_a) * BM; T.b_row0 = (idx / p.tiles_a) * BN;
       T.a_lim = (int)p.rows_a; T.b_lim = (int)p.rows_b;
       T.k_begin = g ? p.offs[g - 1] : 0; T.k_len = p.offs[g] - T.k_begin; T.kb0 = T.k_begin >> 7;
+    }
+  };
+
+  // ---- tile table: the first kTileTable tiles of this workgroup, decoded once by as many lanes
+  // in parallel; the two cursors (loader, MFMAs) then fetch a tile with one LDS read each instead
+  // of redoing the group search and the integer divisions at every tile switch ----
+  constexpr int kTileTable = 48;
+  __shared__ __attribute__((aligned(16))) int s_tiles[kTileTable][8];
+  if (tid < kTileTable) {
+    const int t = t_first + tid * t_step;
+    if (t < t_end) {
+      Tile T;
+      decode_any(t, T);
+      *(int4*)&s_tiles[tid][0] = make_int4(T.a_row0, T.b_row0, T.a_lim, T.b_lim);
+      *(int4*)&s_tiles[tid][4] = make_int4(T.k_begin, T.k_len, T.kb0, T.g);
+    }
+  }
+  __syncthreads();
+  // n = ordinal of the tile in this workgroup's list (t = t_first + n * t_step)
+  auto decode = [&](int n, int t, Tile& T) {
+    if (n < kTileTable) {
+      const int4 a = *(const int4*)&s_tiles[n][0];
+      const int4 b = *(const int4*)&s_tiles[n][4];
+      T.a_row0 = __builtin_amdgcn_readfirstlane(a.x); T.b_row0 = __builtin_amdgcn_readfirstlane(a.y);
+      T.a_lim = __builtin_amdgcn_readfirstlane(a.z); T.b_lim = __builtin_amdgcn_readfirstlane(a.w);
+      T.k_begin = __builtin_amdgcn_readfirstlane(b.x); T.k_len = __builtin_amdgcn_readfirstlane(b.y);
+      T.kb0 = __builtin_amdgcn_readfirstlane(b.z); T.g = __builtin_amdgcn_readfirstlane(b.w);
+    } else {
+      Tile U;
+      decode_any(t, U);
+      T.a_row0 = __builtin_amdgcn_readfirstlane(U.a_row0); T.b_row0 = __builtin_amdgcn_readfirstlane(U.b_row0);
+      T.a_lim = __builtin_amdgcn_readfirstlane(U.a_lim); T.b_lim = __builtin_amdgcn_readfirstlane(U.b_lim);
+      T.k_begin = __builtin_amdgcn_readfirstlane(U.k_begin); T.k_len = __builtin_amdgcn_readfirstlane(U.k_len);
+      T.kb0 = __builtin_amdgcn_readfirstlane(U.kb0); T.g = __builtin_amdgcn_readfirstlane(U.g);
     }
   };
 
@@ -322,14 +359,14 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   // ---- loader: walks (tile, 128-block) pairs ahead of the MFMAs and keeps the LDS ring full ----
   Tile L;
   int lt = t_first - t_step, l_it = 0, l_nk = 0, n_issued = 0;
-  int l_hint = 0, p_hint = 0, c_hint = 0;  // per-cursor group of the last decoded tile (m-grouped mode)
+  int l_n = -1, p_n = -1, c_n = -1;  // per-cursor ordinal of the current tile in this workgroup's list
   v4i rs_b = rs_a, rs_sb = rs_sa;
   uint32_t vs[SPW];  // this wave's per-lane scale offsets (bytes) at step 0 of the loader's tile
   auto issue_stage = [&]() {
     while (l_it >= l_nk) {
       lt += t_step;
       if (lt >= t_end) return;
-      decode(lt, L, l_hint);
+      decode(++l_n, lt, L);
       l_it = 0;
       l_nk = (L.k_len + 127) >> 7;
       rs_b = make_rsrc(p.b + (MODE == GEMM_M_GROUPED ? (int64_t)L.g * p.b_stride_g : 0), (uint32_t)p.b_bytes);
@@ -391,7 +428,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
     while (p_it >= p_nk) {
       pt += t_step;
       if (pt >= t_end) return;
-      decode(pt, Pf, p_hint);
+      decode(++p_n, pt, Pf);
       p_it = 0;
       p_nk = (Pf.k_len + 127) >> 7;
       rs_b_pf = make_rsrc(p.b + (MODE == GEMM_M_GROUPED ? (int64_t)Pf.g * p.b_stride_g : 0), (uint32_t)p.b_bytes);
@@ -439,7 +476,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   Tile C;
 #pragma unroll 1
   for (int t = t_first; t < t_end; t += t_step) {
-    decode(t, C, c_hint);
+    decode(++c_n, t, C);
     const int nk = (C.k_len + 127) >> 7;
     // Waves whose whole row range lies past the end of a ragged group skip the MFMAs (they still
     // take part in the loads and barriers).
