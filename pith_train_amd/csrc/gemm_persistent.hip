@@ -118,9 +118,9 @@ __device__ __forceinline__ void store_staged_bf16(const v16f& a, __amdgpu_buffer
     const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, false);
     *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = __builtin_amdgcn_perm(nb, pk, sel);
   }
-  // the reads below alias the writes above: keep the compiler from reordering them and let the
-  // writes land first
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  // the reads below alias the writes above: keep the compiler from reordering them (the LDS
+  // executes one wave's operations in order, so no counter wait is needed)
+  asm volatile("" ::: "memory");
   const uint8_t* rd = stg + (lane >> 2) * 64 + (lane & 3) * 16;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
@@ -154,7 +154,7 @@ __device__ __forceinline__ void store_staged_bf16_rows(const v16f& a, __amdgpu_b
     const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, false);
     *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = __builtin_amdgcn_perm(nb, pk, sel);
   }
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  asm volatile("" ::: "memory");  // compiler fence only: same-wave LDS operations execute in order
   const uint8_t* rd = stg + (lane >> 2) * 64 + (lane & 3) * 16;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
