@@ -129,18 +129,23 @@ class GptOssExperts(nn.Module):
             cache[name] = fp8cast_blockwise_transpose_batched(weight)
         return cache[name]
 
-    def _group_linear(self, x, weight, name, offs, ks, ks_tensor, group_indices_):
+    def _group_linear(self, x, weight, name, offs, ks, ks_tensor, group_indices_, in_rows=None):
         if x.shape[0] == 0:
             return x @ weight[0].transpose(-2, -1)
         if training.fp8:
             return FP8GroupedLinearFunc.apply(
-                x, weight, offs, ks, ks_tensor, self._quantized_weight(name, weight), group_indices_
+                x, weight, offs, ks, ks_tensor, self._quantized_weight(name, weight), group_indices_, in_rows
             )
+        assert in_rows is None, "row maps need the FP8 layers"
         return GroupedLinearFunc.apply(x, weight, offs)
 
-    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None):
-        group_ids = group_indices(grouped_mm_offs, x.shape[0], torch.int64)
-        gate_up = self._group_linear(x, self.gate_up_proj, "gate_up_proj", grouped_mm_offs, ks, ks_tensor, None)
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None):
+        """``row_map`` (extension, FP8 only): the scatter's int32 source-row map; ``x`` is then the
+        un-permuted token tensor and the first quantisation gathers its rows (the result stays in
+        the grouped layout: the per-group bias gradients are sums over contiguous row ranges)."""
+        M = x.shape[0] if row_map is None else row_map.shape[0]
+        group_ids = group_indices(grouped_mm_offs, M, torch.int64)
+        gate_up = self._group_linear(x, self.gate_up_proj, "gate_up_proj", grouped_mm_offs, ks, ks_tensor, None, row_map)
         gate_up = indexed_bias_add(gate_up, self.gate_up_proj_bias, group_ids, grouped_mm_offs)
         activated = clamped_swiglu(gate_up, 1.702, self.swiglu_limit)
         out = self._group_linear(activated, self.down_proj, "down_proj", grouped_mm_offs, ks, ks_tensor, None)
@@ -169,6 +174,13 @@ def forward_stage3(experts: nn.Module, gathered_tokens, expert_idxs, experts_per
         _, grouped_mm_offs, ks, ks_tensor, src_of = group_rows_with_sizes(
             expert_idxs, experts_per_rank, device=gathered_tokens.device)
         return experts(gathered_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, row_map=src_of)
+    if (fuse_permute and expand_idx is None and training.fp8 and expert_idxs.shape[0] > 0
+            and isinstance(experts, GptOssExperts)):
+        # input side only: the output keeps the grouped layout for the per-group bias sums
+        reverse_shuffle_idxs, grouped_mm_offs, ks, ks_tensor, src_of = group_rows_with_sizes(
+            expert_idxs, experts_per_rank, device=gathered_tokens.device)
+        outs = experts(gathered_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, row_map=src_of)
+        return padded_index_gather(outs, reverse_shuffle_idxs)
     pre = None
     if expand_idx is not None:
         if fuse_expand:
