@@ -136,7 +136,9 @@ class GemmTimer:
                 a.record()
                 orig(name, *args)
                 b.record()
-                timer.records.append((name, a, b))
+                # rows x columns x reduction as the entry point takes them (the three int64 sizes)
+                sizes = {"pt_gemm_nt_dense": args[6:9], "pt_gemm_k_grouped_wgrad": args[9:12]}.get(name, args[8:11])
+                timer.records.append((name, a, b, "x".join(str(int(v)) for v in sizes)))
             else:
                 orig(name, *args)
 
@@ -146,11 +148,20 @@ class GemmTimer:
 
     def summary(self):
         out = {}
-        for name, a, b in self.records:
+        for name, a, b, _ in self.records:
             d = out.setdefault(name, [0.0, 0])
             d[0] += a.elapsed_time(b)
             d[1] += 1
         return {k: {"ms_total": v[0], "launches": v[1]} for k, v in out.items()}
+
+    def by_shape(self, steps):
+        """Average duration in microseconds of one launch per (entry point, M x N x K) of a step."""
+        out = {}
+        for name, a, b, shape in self.records:
+            d = out.setdefault(f"{name.replace('pt_gemm_', '')} {shape}", [0.0, 0])
+            d[0] += a.elapsed_time(b)
+            d[1] += 1
+        return {k: {"us": round(v[0] / v[1] * 1e3, 1), "launches_per_step": v[1] / max(steps, 1)} for k, v in out.items()}
 
 
 def hbm_kernel_report(H, I, E, rows, eidx):
@@ -396,7 +407,7 @@ def main():
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "fp8_gemm_nt_persistent_kernel (every GEMM launch of the step: fwd, dgrad, wgrad)",
+            "kernel": "fp8_gemm_nt_persistent_kernel / fp8_gemm_nt_pipelined_kernel (every GEMM launch of the step: fwd, dgrad, wgrad; the library picks the main loop per shape)",
             "achieved": achieved,
             "peak": FP8_DENSE_PEAK_TFLOPS,
             "unit": "TFLOP/s",
@@ -407,6 +418,7 @@ def main():
             "launches_per_step": gemm_launches / max(args.steps, 1),
             "gemm_ms_per_step": gemm_ms / max(args.steps, 1),
             "per_entry_point_ms_per_step": {k2: v["ms_total"] / args.steps for k2, v in gs.items()},
+            "per_shape": timer.by_shape(args.steps),
         },
         **extra,
     }

@@ -140,6 +140,15 @@ int pt_gemm_k_grouped_wgrad(const void* dy_t_fp8, const float* dy_scale, const v
                             const int32_t* offs, int32_t num_groups, int64_t M, int64_t N,
                             int64_t K, pt_stream_t stream);
 
+/* Which GEMM kernel the three entry points above launch: "auto" (or NULL: per call from the
+ * shape; the default unless the environment variable PT_GEMM_IMPL names one of the others),
+ * "p0" persistent kernel with the two-phase main loop, "q0" / "q1" persistent kernel with the
+ * software-pipelined main loop (8 / 4 waves per workgroup), "t" one 128x128 tile per workgroup.
+ * Every choice computes the same function; this exists for measurements and for tests that
+ * cover each kernel.  Process-wide, not synchronised with concurrent GEMM calls.
+ * No counterpart in the reference (DeepGEMM selects its kernels internally). */
+int pt_gemm_select_kernel(const char* name);
+
 /* ------------------------------------------------------------------------------------------
  * Routing-driven permute / unpermute.  Replace pithtrain/operators/token_scatter.py.
  * ------------------------------------------------------------------------------------------ */

@@ -17,6 +17,7 @@
 #include "common.h"
 #include "gemm_args.h"
 #include <stdlib.h>
+#include <string.h>
 
 namespace pt {
 
@@ -260,34 +261,66 @@ static int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   return check_launch("fp8_gemm_nt_kernel");
 }
 
-// PT_GEMM_IMPL selects the kernel for experiments: "tile" = one tile per workgroup (128x128),
-// "p0" / "p1" / "p2" = persistent kernel variants.  Default: persistent 256x256.
+// PT_GEMM_IMPL overrides the choice of kernel for measurements: "t" = one 128x128 tile per
+// workgroup, "p0" = persistent two-phase kernel, "q0" / "q1" = persistent software-pipelined kernel
+// (8 / 4 waves).  Unset: chosen per call from the shape (below).
+enum { IMPL_UNSET = -3, IMPL_AUTO = -2, IMPL_TILE = -1, IMPL_PIPELINED = 100 };
+static int g_impl = IMPL_UNSET;
+static bool parse_impl(const char* e, int& impl) {
+  if (!e || !*e || !strcmp(e, "auto")) impl = IMPL_AUTO;
+  else if (!strcmp(e, "t")) impl = IMPL_TILE;
+  else if (!strcmp(e, "p0")) impl = 0;
+  else if (!strcmp(e, "q0") || !strcmp(e, "q1")) impl = IMPL_PIPELINED + (e[1] - '0');
+  else return false;
+  return true;
+}
 static int gemm_impl() {
-  static int impl = -2;
-  if (impl == -2) {
-    const char* e = getenv("PT_GEMM_IMPL");
-    if (!e || !*e) impl = 0;
-    else if (e[0] == 't') impl = -1;
-    else if (e[0] == 'p') impl = atoi(e + 1);
-    else impl = 0;
+  if (g_impl == IMPL_UNSET) {
+    int impl;
+    g_impl = parse_impl(getenv("PT_GEMM_IMPL"), impl) ? impl : IMPL_AUTO;
   }
-  return impl;
+  return g_impl;
+}
+
+// The software-pipelined loop overlaps one wave's LDS reads with its own MFMAs but pays a fixed
+// fill/drain of one 128-block per tile, and its tile switch is slower; the two-phase loop is the
+// better one when a tile's reduction is short or the groups are small (few row tiles per group:
+// many half-empty tiles and frequent changes of the b operand).  Crossovers measured on MI355X
+// inside a training step (operands freshly written, i.e. partly cache-resident):
+//   dense      pipelined from K = 512 on (+5 % at 512, +13..20 % from 2048 on)
+//   m-grouped  pipelined for >= 1536 rows per group and K >= 2048 (+3..13 %); below, -2..-9 %
+//   k-grouped  pipelined for >= 6 blocks of 128 rows per group (+0..6 %); at 4.5 blocks, -5..-9 %
+static bool prefer_pipelined(const GemmArgs& g) {
+  switch (g.mode) {
+    case GEMM_DENSE: return g.red >= 512;
+    case GEMM_M_GROUPED: return g.G > 0 && g.red >= 2048 && g.rows_a >= (int64_t)g.G * 1536;
+    default: return g.G > 0 && g.red >= (int64_t)g.G * 128 * 6;
+  }
 }
 
 static int dispatch_gemm(const GemmArgs& g, hipStream_t stream) {
   const int impl = gemm_impl();
-  // the persistent kernel addresses operands through 32-bit buffer offsets
+  // the persistent kernels address operands through 32-bit buffer offsets
   const int64_t lim = (1ll << 31) - 1;
   const bool fits = g.a_bytes < lim && g.b_bytes < lim && g.sa_bytes < lim && g.sb_bytes < lim && g.rows_a < lim &&
                     g.rows_b < lim && g.red < lim;
-  PT_REQUIRE(!g.out_row_index || (impl >= 0 && fits), "gemm: scattered output rows need the persistent kernel");
-  if (impl < 0 || !fits) return launch_gemm<128, 128, 2, 2>(g, stream);
+  PT_REQUIRE(!g.out_row_index || (impl != IMPL_TILE && fits), "gemm: scattered output rows need the persistent kernel");
+  if (impl == IMPL_TILE || !fits) return launch_gemm<128, 128, 2, 2>(g, stream);
+  if (impl == IMPL_AUTO) return prefer_pipelined(g) ? launch_gemm_pipelined(g, 0, stream) : launch_gemm_persistent(g, 0, stream);
+  if (impl >= IMPL_PIPELINED) return launch_gemm_pipelined(g, impl - IMPL_PIPELINED, stream);
   return launch_gemm_persistent(g, impl, stream);
 }
 
 }  // namespace pt
 
 using namespace pt;
+
+extern "C" int pt_gemm_select_kernel(const char* name) {
+  int impl;
+  PT_REQUIRE(parse_impl(name, impl), "gemm_select_kernel: unknown kernel '%s' (auto, p0, q0, q1, t)", name);
+  g_impl = impl;
+  return PT_OK;
+}
 
 static bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 

@@ -20,13 +20,14 @@ struct GemmArgs {
   int tiles_a, tiles_b;                   // tile counts along rows_a / rows_b
   int64_t a_bytes, b_bytes, sa_bytes, sb_bytes;  // extents of a, one group of b, and their scale arrays
   int64_t total_tiles;
-  int pf_dist;                            // L2 prefetch distance in 128-blocks beyond the LDS ring
   const int32_t* out_row_index;           // m-grouped only: output row of result row r (negative: dropped); null = identity
   int64_t out_rows;                       // rows of the output when out_row_index is given
 };
 
 
-// persistent-kernel launcher (gemm_persistent.hip); variant selects the tile shape
+// persistent kernel with the two-phase main loop (gemm_persistent.hip); variant selects the wave layout
 int launch_gemm_persistent(const GemmArgs& a, int variant, hipStream_t stream);
+// persistent kernel with the software-pipelined main loop (gemm_pipelined.hip)
+int launch_gemm_pipelined(const GemmArgs& a, int variant, hipStream_t stream);
 
 }  // namespace pt

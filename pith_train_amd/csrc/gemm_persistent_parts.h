@@ -1,0 +1,363 @@
+// Parts shared by the two persistent FP8 GEMM kernels (two-phase and software-pipelined main
+// loops): buffer descriptors and direct-to-LDS loads, the work list (group scan, tile geometry),
+// the result stores, and the launch of one workgroup per CU.
+#pragma once
+#include "common.h"
+#include "gemm_args.h"
+#include <stdlib.h>
+
+namespace pt {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+static constexpr int kMaxGroupsGemm = 2048;
+static constexpr uint32_t kOob = 0x80000000u;  // per-lane offset that is out of range for every descriptor used here
+static constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
+
+// Raw buffer descriptor over [base, base + bytes) for the inline-assembly loads.
+__device__ __forceinline__ v4i make_rsrc(const void* base, uint32_t bytes) {
+  const uint64_t a = (uint64_t)(uintptr_t)base;
+  v4i r;
+  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+  r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((a >> 32) & 0xFFFF));
+  r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+  r[3] = kRsrcFlags;
+  return r;
+}
+
+// Direct-to-LDS buffer loads: address = base + voff (per lane) + soff (uniform); lane l's data lands
+// at lds_off + 16*l (dwordx4) or lds_off + 4*l (dword).  lds_off is a wave-uniform LDS byte address.
+__device__ __forceinline__ void dma16(v4i rsrc, uint32_t voff, uint32_t soff, uint32_t lds_off) {
+  soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);  // uniform by construction; pin them to SGPRs
+  lds_off = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_off);
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff),
+               "s"(lds_off)
+               : "memory");
+}
+__device__ __forceinline__ void dma4(v4i rsrc, uint32_t voff, uint32_t soff, uint32_t lds_off) {
+  soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
+  lds_off = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_off);
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff),
+               "s"(lds_off)
+               : "memory");
+}
+__device__ __forceinline__ void wait_all_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+  const bf16x2 h = __builtin_convertvector(f32x2{lo, hi}, bf16x2);
+  return __builtin_bit_cast(uint32_t, h);
+}
+
+// ---- epilogue of one 32x32 accumulator tile.  The lane holds column (lane&31) and rows
+// 8*(v/4) + 4*(lane>>5) + (v&3).  voff is the lane's byte offset inside the tile (kOob if its
+// column is out of range); soff the uniform byte offset of the tile's row 0, column 0; pitch the
+// row pitch in bytes. ----
+__device__ __forceinline__ void store_f32(const v16f& a, __amdgpu_buffer_rsrc_t out, uint32_t voff, uint32_t soff,
+                                          uint32_t pitch, bool accumulate) {
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const uint32_t s = soff + (8 * (v >> 2) + (v & 3)) * pitch;
+    float x = a[v];
+    if (accumulate) x += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(out, voff, s, 0));
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, x), out, voff, s, 0);
+  }
+}
+// bf16: lanes 2c and 2c+1 trade one value of each register pair so that each stores two adjacent
+// columns of one row as a dword (the odd lane writes one row below the even lane; voff already
+// says so).  Needs an even row pitch in elements.
+__device__ __forceinline__ void store_pairs_bf16(const v16f& a, __amdgpu_buffer_rsrc_t out, uint32_t voff, uint32_t soff,
+                                                 uint32_t pitch, bool accumulate, bool odd) {
+#pragma unroll
+  for (int v = 0; v < 16; v += 2) {
+    const float x0 = a[v], x1 = a[v + 1];
+    const float send = odd ? x0 : x1;
+    const float recv = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send), 0xB1, 0xF, 0xF, false));
+    const uint32_t s = soff + (8 * (v >> 2) + (v & 3)) * pitch;
+    // round the GEMM result to bf16 first, then add: the two roundings of `grad += wgrad.to(bf16)`
+    uint32_t w = odd ? pack2_bf16(recv, x1) : pack2_bf16(x0, recv);
+    if (accumulate) {
+      const uint32_t old = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(out, voff, s, 0);
+      w = pack2_bf16(bf16_lo(old) + bf16_lo(w), bf16_hi(old) + bf16_hi(w));
+    }
+    __builtin_amdgcn_raw_buffer_store_b32((int)w, out, voff, s, 0);
+  }
+}
+// bf16 through a per-wave LDS staging tile (32 rows x 64 B): the accumulator layout (a lane owns
+// one column) is turned into rows, so that every lane stores 16 contiguous bytes and one store
+// instruction covers 16 rows x 64 B.  The memory pipeline spends the same time on a 4-byte and a
+// 16-byte store instruction, so this is a quarter of the store issue time of store_pairs_bf16.
+// Only this wave touches its staging tile, so a counter wait between the phases is enough.
+// voff: lane's byte offset (row lane/4, 16-byte chunk lane%4) or kOob; soff: tile row 0, column 0.
+__device__ __forceinline__ void store_staged_bf16(const v16f& a, __amdgpu_buffer_rsrc_t out, uint8_t* stg, uint32_t voff,
+                                                  uint32_t soff, uint32_t pitch, bool accumulate, int lane) {
+  const bool odd = lane & 1;
+  uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 64 + ((lane & 31) >> 1) * 4;
+  // p = (row r | row r+1) of the lane's column; the even lane of a pair takes both low halves (row r,
+  // columns c and c+1), the odd lane both high halves (row r+1): one byte permute of own and neighbour
+  const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
+#pragma unroll
+  for (int v = 0; v < 16; v += 2) {
+    const uint32_t pk = pack2_bf16(a[v], a[v + 1]);
+    const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, false);
+    *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = __builtin_amdgcn_perm(nb, pk, sel);
+  }
+  // the reads below alias the writes above: keep the compiler from reordering them (the LDS
+  // executes one wave's operations in order, so no counter wait is needed)
+  asm volatile("" ::: "memory");
+  const uint8_t* rd = stg + (lane >> 2) * 64 + (lane & 3) * 16;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    v4i w = *(const v4i*)(rd + h * 1024);
+    const uint32_t s = soff + h * 16 * pitch;
+    if (accumulate) {
+      const v4i old = __builtin_amdgcn_raw_buffer_load_b128(out, voff, s, 0);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        w[q] = (int)pack2_bf16(bf16_lo((uint32_t)old[q]) + bf16_lo((uint32_t)w[q]), bf16_hi((uint32_t)old[q]) + bf16_hi((uint32_t)w[q]));
+    }
+    __builtin_amdgcn_raw_buffer_store_b128(w, out, voff, s, 0);
+    // A 16-byte store reads its data registers for a few cycles after it issues; the compiler
+    // only guards that window for stores without a scalar offset, so hold the registers here.
+    asm volatile("s_nop 4" ::"v"(w) : "memory");
+  }
+}
+// As store_staged_bf16 with an arbitrary output row per lane: voff0 / voff1 are the lane's byte
+// offsets (row start + 16-byte chunk, or kOob) for tile rows lane/4 and 16 + lane/4; soff the
+// column offset in bytes.
+__device__ __forceinline__ void store_staged_bf16_rows(const v16f& a, __amdgpu_buffer_rsrc_t out, uint8_t* stg, uint32_t voff0,
+                                                       uint32_t voff1, uint32_t soff, int lane) {
+  const bool odd = lane & 1;
+  uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 64 + ((lane & 31) >> 1) * 4;
+  // p = (row r | row r+1) of the lane's column; the even lane of a pair takes both low halves (row r,
+  // columns c and c+1), the odd lane both high halves (row r+1): one byte permute of own and neighbour
+  const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
+#pragma unroll
+  for (int v = 0; v < 16; v += 2) {
+    const uint32_t pk = pack2_bf16(a[v], a[v + 1]);
+    const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, false);
+    *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = __builtin_amdgcn_perm(nb, pk, sel);
+  }
+  asm volatile("" ::: "memory");  // compiler fence only: same-wave LDS operations execute in order
+  const uint8_t* rd = stg + (lane >> 2) * 64 + (lane & 3) * 16;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const v4i w = *(const v4i*)(rd + h * 1024);
+    __builtin_amdgcn_raw_buffer_store_b128(w, out, h ? voff1 : voff0, soff, 0);
+    asm volatile("s_nop 4" ::"v"(w) : "memory");  // see store_staged_bf16
+  }
+}
+__device__ __forceinline__ void store_single_bf16(const v16f& a, __amdgpu_buffer_rsrc_t out, uint32_t voff, uint32_t soff,
+                                                  uint32_t pitch, bool accumulate) {
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const uint32_t s = soff + (8 * (v >> 2) + (v & 3)) * pitch;
+    uint32_t r = f32_to_bf16_bits(a[v]);
+    if (accumulate) {
+      const uint32_t old = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(out, voff, s, 0);
+      r = f32_to_bf16_bits(bf16_bits_to_f32(old) + bf16_bits_to_f32(r));
+    }
+    __builtin_amdgcn_raw_buffer_store_b16((short)r, out, voff, s, 0);
+  }
+}
+
+// One tile of the work list; everything is wave-uniform (SGPRs).
+struct Tile {
+  int a_row0, b_row0, a_lim, b_lim, k_begin, k_len, kb0, g;
+};
+
+// s_pref[g] = number of BM-row tiles of groups < g (s_pref[G] = their total), from the cumulative
+// group ends in p.offs; computed by the first wave, followed by a workgroup barrier.
+template <int BM>
+__device__ __forceinline__ void scan_group_tiles(const GemmArgs& p, int* s_pref, int tid, int lane) {
+  if (tid < 64) {
+    const int per = (p.G + 63) / 64;
+    const int g0 = tid * per;
+    int sum = 0;
+    for (int q = 0; q < per; ++q) {
+      const int g = g0 + q;
+      if (g < p.G) sum += (p.offs[g] - (g ? p.offs[g - 1] : 0) + BM - 1) / BM;
+    }
+    int incl = sum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int y = __shfl_up(incl, d);
+      if (lane >= d) incl += y;
+    }
+    int run = incl - sum;
+    for (int q = 0; q < per; ++q) {
+      const int g = g0 + q;
+      if (g < p.G) {
+        s_pref[g] = run;
+        run += (p.offs[g] - (g ? p.offs[g - 1] : 0) + BM - 1) / BM;
+      }
+    }
+    if (tid == 63) s_pref[p.G] = incl;
+  }
+  __syncthreads();
+}
+
+// Geometry of logical tile t; plain per-lane arithmetic (every lane may ask for a different t).
+template <int MODE, int BM, int BN>
+__device__ __forceinline__ void decode_tile(const GemmArgs& p, const int* s_pref, int t, Tile& T) {
+  if (MODE == GEMM_DENSE) {
+    T.g = 0;
+    // The 32 CUs of an XCD work on 32 consecutive logical tiles at a time; laying those out as
+    // a 4 x 8 block of the output makes them share 4 a-tiles and 8 b-tiles in that XCD's L2
+    // instead of 32 a-tiles and 1 b-tile.
+    int ta, tb;
+    const int full_a = p.tiles_a & ~3, full_b = p.tiles_b & ~7;
+    const int nblk = (full_a >> 2) * (full_b >> 3);
+    if (t < nblk * 32) {
+      const int blk = t >> 5, in = t & 31;
+      ta = (blk % (full_a >> 2)) * 4 + (in & 3);
+      tb = (blk / (full_a >> 2)) * 8 + (in >> 2);
+    } else {  // ragged fringe: remaining columns of tiles, then remaining rows
+      const int r = t - nblk * 32;
+      const int fringe_b = p.tiles_b - full_b;  // extra b-tiles, all a-tiles
+      if (r < fringe_b * p.tiles_a) { ta = r % p.tiles_a; tb = full_b + r / p.tiles_a; }
+      else { const int r2 = r - fringe_b * p.tiles_a; ta = full_a + r2 % (p.tiles_a - full_a); tb = r2 / (p.tiles_a - full_a); }
+    }
+    T.a_row0 = ta * BM; T.b_row0 = tb * BN;
+    T.a_lim = (int)p.rows_a; T.b_lim = (int)p.rows_b; T.k_begin = 0; T.k_len = (int)p.red; T.kb0 = 0;
+  } else if (MODE == GEMM_M_GROUPED) {
+    const int q = t / p.tiles_b;
+    int lo = 1, hi = p.G;  // first j in [1, G] with s_pref[j] > q
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (s_pref[mid] > q) hi = mid; else lo = mid + 1;
+    }
+    const int g = lo - 1;
+    const int pg = s_pref[g], pg1 = s_pref[g + 1];
+    const int gs = g ? p.offs[g - 1] : 0;
+    const int m_tiles = pg1 - pg;
+    const int idx = t - pg * p.tiles_b;
+    T.g = g;
+    T.a_row0 = gs + (idx % m_tiles) * BM; T.b_row0 = (idx / m_tiles) * BN;
+    T.a_lim = p.offs[g]; T.b_lim = (int)p.rows_b; T.k_begin = 0; T.k_len = (int)p.red; T.kb0 = 0;
+  } else {
+    const int per_g = p.tiles_a * p.tiles_b;
+    const int g = t / per_g;
+    const int idx = t % per_g;
+    T.g = g;
+    T.a_row0 = (idx % p.tiles_a) * BM; T.b_row0 = (idx / p.tiles_a) * BN;
+    T.a_lim = (int)p.rows_a; T.b_lim = (int)p.rows_b;
+    T.k_begin = g ? p.offs[g - 1] : 0; T.k_len = p.offs[g] - T.k_begin; T.kb0 = T.k_begin >> 7;
+  }
+}
+
+// Writes one wave's TM x TN blocks of 32 x 32 results of tile T (rows wm0.., columns wn0.. of the
+// tile).  `stg` is the wave's 2 KiB LDS staging area.  PIN: the accumulators were produced by
+// inline-assembly MFMAs and live in the accumulation registers; each block is handed to the
+// compiler only right before its store, so that it is copied out one block at a time.
+template <int MODE, int TM, int TN, bool ACC, bool PIN>
+__device__ __forceinline__ void store_tile(v16f (&acc)[TM][TN], const GemmArgs& p, const Tile& T, int wm0, int wn0, int lane,
+                                           uint8_t* stg) {
+  const uint32_t esz = p.out_dtype == PT_F32 ? 4 : 2;
+  const uint32_t pitch = (uint32_t)p.ldo * esz;
+  const bool pair_ok = p.out_dtype != PT_F32 && (p.ldo & 1) == 0 && (((uintptr_t)p.out) & 3) == 0;
+  const bool wide_ok = p.out_dtype != PT_F32 && (p.ldo & 7) == 0 && (((uintptr_t)p.out) & 15) == 0 &&
+                       (MODE != GEMM_K_GROUPED || (p.out_stride_g & 7) == 0);
+  // The descriptor ends after the tile's last valid row: stores to ragged rows are dropped.
+  char* outp = (char*)p.out + (MODE == GEMM_K_GROUPED ? (int64_t)T.g * p.out_stride_g * esz : 0);
+  const __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(outp, 0, (int)((uint32_t)T.a_lim * pitch), kRsrcFlags);
+  const uint32_t s_tile = (uint32_t)(T.a_row0 + wm0) * pitch + (uint32_t)(T.b_row0 + wn0) * esz;
+  const int colw = T.b_row0 + wn0 + (lane & 31);
+  if (MODE == GEMM_M_GROUPED && p.out_row_index) {
+    // Result row r goes to output row out_row_index[r] (the un-permute folded into the store);
+    // rows of the group's padding map to a negative index and are dropped.
+    const __amdgpu_buffer_rsrc_t rs_sc = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, (int)((uint32_t)p.out_rows * pitch), kRsrcFlags);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      uint32_t vrow[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int r = T.a_row0 + wm0 + i * 32 + h * 16 + (lane >> 2);
+        const int dst = r < T.a_lim ? p.out_row_index[r] : -1;
+        vrow[h] = dst >= 0 ? (uint32_t)dst * pitch + (uint32_t)(lane & 3) * 16 : kOob;
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int colc = T.b_row0 + wn0 + j * 32 + (lane & 3) * 8;
+        const bool col_ok = colc < T.b_lim;
+        if constexpr (PIN) if constexpr (PIN) asm volatile("" : "+a"(acc[i][j]));
+        store_staged_bf16_rows(acc[i][j], rs_sc, stg, col_ok ? vrow[0] : kOob, col_ok ? vrow[1] : kOob,
+                               (uint32_t)(T.b_row0 + wn0 + j * 32) * 2, lane);
+      }
+    }
+  } else if (p.out_dtype != PT_F32 && wide_ok && (T.b_lim & 7) == 0) {
+    // rows first, then the column blocks of a row band back to back: adjacent 64-byte halves of
+    // a cache line are written by consecutive instructions
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int colc = T.b_row0 + wn0 + j * 32 + (lane & 3) * 8;
+        const uint32_t voff = colc < T.b_lim ? (uint32_t)(lane >> 2) * pitch + (uint32_t)(lane & 3) * 16 : kOob;
+        if constexpr (PIN) asm volatile("" : "+a"(acc[i][j]));
+        store_staged_bf16(acc[i][j], rs_out, stg, voff, s_tile + i * 32 * pitch + j * 64, pitch, ACC, lane);
+      }
+  } else if (p.out_dtype != PT_F32 && pair_ok && (T.b_lim & 1) == 0) {
+    const bool odd = lane & 1;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const uint32_t voff = colw + j * 32 < T.b_lim ? (uint32_t)(4 * (lane >> 5) + odd) * pitch + (uint32_t)(((lane & 31) & ~1) + j * 32) * 2 : kOob;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) { if constexpr (PIN) asm volatile("" : "+a"(acc[i][j])); store_pairs_bf16(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC, odd); }
+    }
+  } else if (p.out_dtype == PT_F32) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const uint32_t voff = colw + j * 32 < T.b_lim ? (uint32_t)(4 * (lane >> 5)) * pitch + (uint32_t)((lane & 31) + j * 32) * 4 : kOob;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) { if constexpr (PIN) asm volatile("" : "+a"(acc[i][j])); store_f32(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC); }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const uint32_t voff = colw + j * 32 < T.b_lim ? (uint32_t)(4 * (lane >> 5)) * pitch + (uint32_t)((lane & 31) + j * 32) * 2 : kOob;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) { if constexpr (PIN) asm volatile("" : "+a"(acc[i][j])); store_single_bf16(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC); }
+    }
+  }
+}
+
+// One workgroup per CU (fewer when there are fewer tiles), in multiples of the 8 XCDs.  `upper` is
+// an upper bound of the number of tiles.
+template <class Kernel>
+static int launch_persistent_grid(Kernel kernel, const char* name, const GemmArgs& a, int64_t upper, int threads, size_t lds,
+                                  bool& attr_set, hipStream_t stream) {
+  static int num_cus = 0;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { set_error("gemm: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e)); return PT_ERR_LAUNCH; }
+    attr_set = true;
+  }
+  if (num_cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    num_cus = n;
+  }
+  if (upper == 0) return PT_OK;
+  PT_REQUIRE(upper < (1ll << 30), "gemm: too many tiles");
+  int64_t blocks = (num_cus + 7) / 8 * 8;
+  if (upper < blocks) blocks = (upper + 7) / 8 * 8;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(threads), lds, stream, a);
+  return check_launch(name);
+}
+
+// Fills the tile counts of `a` for BM x BN tiles and returns an upper bound of the number of tiles
+// (exact except in the m-grouped mode, where the kernel counts them from the group sizes).
+static inline int64_t plan_tiles(GemmArgs& a, int BM, int BN) {
+  a.tiles_a = (int)cdiv(a.rows_a, BM);
+  a.tiles_b = (int)cdiv(a.rows_b, BN);
+  if (a.mode == GEMM_DENSE) return a.total_tiles = (int64_t)a.tiles_a * a.tiles_b;
+  if (a.mode == GEMM_K_GROUPED) return a.total_tiles = (int64_t)a.tiles_a * a.tiles_b * a.G;
+  return ((a.rows_a / 128 + a.G) / 2 + 1) * a.tiles_b;
+}
+
+}  // namespace pt

@@ -18,6 +18,16 @@ pytestmark = pytest.mark.gpu
 REL = 1e-2
 
 
+@pytest.fixture(autouse=True, params=["auto", "p0", "q0", "t"])
+def gemm_kernel(request):
+    """Every test runs once per GEMM kernel of the library (and once with the library's own choice)."""
+    from pith_train_amd import _lib
+
+    _lib.call("pt_gemm_select_kernel", request.param.encode())
+    yield request.param
+    _lib.call("pt_gemm_select_kernel", None)
+
+
 def _check(got, ref, what):
     got = got.float().cpu().double()
     ref = ref.double()
@@ -81,6 +91,7 @@ GROUPED = [
     ([256] * 8, 512, 256),
     ([512, 640, 128, 0, 384], 1536, 2048),
     ([300, 200], 2880, 2880),
+    ([1536, 1700], 256, 2048),  # large groups + long reduction: the pipelined loop by the library's own choice
 ]
 
 
@@ -102,6 +113,41 @@ def test_m_grouped_nt(sizes, N, K):
     out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
     m_grouped_fp8_gemm_nt((a.cuda(), sa.cuda()), (b.cuda(), sb.cuda()), out, offs.cuda())
     _check(out, ref, f"m-grouped {sizes} N={N} K={K}")
+
+
+@pytest.mark.parametrize("sizes,N,K", GROUPED)
+def test_m_grouped_nt_scattered_rows(sizes, N, K, gemm_kernel):
+    """The un-permute folded into the store: result row r lands in output row out_rows[r]; rows of
+    a group's padding (negative index) are dropped and rows nobody maps to stay untouched."""
+    from pith_train_amd.operators.grouped_linear import m_grouped_fp8_gemm_nt
+
+    if gemm_kernel == "t":
+        pytest.skip("the tile-per-workgroup kernel has no scattered store (the library refuses it)")
+    ks, offs = _groups(sizes)
+    M, Gn = int(offs[-1]), len(sizes)
+    x = _rand((M, K), M + K + 17)
+    w = _rand((Gn, N, K), N + K + 5, 0.02)
+    a, sa, _, _ = Q.fp8cast_rowwise_colwise(x)
+    b, sb, _, _ = Q.fp8cast_blockwise_transpose_batched(w)
+    ref = G.gemm_m_grouped_nt(a, sa, b, sb, offs, torch.float64)
+    real = torch.zeros(M, dtype=torch.bool)
+    start = 0
+    for s_, k_ in zip(sizes, ks.tolist()):
+        real[start : start + s_] = True
+        start += k_
+    n_real = int(real.sum())
+    out_m = n_real + 3  # three rows that no result row maps to
+    g = torch.Generator().manual_seed(M)
+    dst = torch.randperm(out_m, generator=g)[:n_real].to(torch.int32)
+    out_rows = torch.full((M,), -1, dtype=torch.int32)
+    out_rows[real] = dst
+    out = torch.full((out_m, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    m_grouped_fp8_gemm_nt((a.cuda(), sa.cuda()), (b.cuda(), sb.cuda()), out, offs.cuda(), out_rows.cuda())
+    out = out.cpu()
+    _check(out[dst.long()], ref[real], f"m-grouped scattered {sizes} N={N} K={K}")
+    untouched = torch.ones(out_m, dtype=torch.bool)
+    untouched[dst.long()] = False
+    assert (out[untouched] == 7.0).all()
 
 
 @pytest.mark.parametrize("sizes,N,K", GROUPED)
