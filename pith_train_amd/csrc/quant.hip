@@ -9,6 +9,7 @@
 // through an XOR-swizzled LDS tile so that global stores are 16 bytes wide and 128-byte
 // contiguous per 8 lanes.  The kernel is HBM-bound: 2 (or 4) bytes in, 2 bytes out per element.
 #include "common.h"
+#include <type_traits>
 
 namespace pt {
 
@@ -101,22 +102,45 @@ template <> struct Frag<float> {
 
 enum { PRO_NONE = 0, PRO_SILU_FWD = 1, PRO_SILU_BWD = 2, PRO_SILU_BWD_PAIR = 3 };  // what the tile is computed from
 
-template <typename T, int AM, int BMODE, int BL, int BS, int PRO = PRO_NONE>
-__global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
-  __shared__ float s_colmax[4][128];
-  __shared__ float s_blk[4];
-  __shared__ __attribute__((aligned(16))) uint8_t s_t[128 * 128];
+// ---- packed-bf16 arithmetic of the interior-tile path -------------------------------------------
+// |x| of a bf16 is its low 15 bits, and for non-negative floats the integer order of the bits is
+// the numeric order: an amax over packed pairs is one AND and one 16-bit packed integer max per two
+// elements, with no unpacking.  (A NaN input compares as larger than everything here, while the
+// float max of the edge-tile path skips it; the results agree for every finite and infinite input.)
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_abs(uint32_t w) { return w & 0x7FFF7FFFu; }
+__device__ __forceinline__ uint32_t pk_umax(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
+// the larger half of a packed pair, as the fp32 with those bf16 bits
+__device__ __forceinline__ float pk_hmax_f32(uint32_t m) {
+  const uint32_t lo = m << 16, hi = m & 0xFFFF0000u;
+  return __uint_as_float(lo > hi ? lo : hi);
+}
+// Two packed bf16 -> two e4m3 bytes of x / scale (scale a power of two, so the quotient is exact and
+// equals x * (1/scale)), placed in the low or high half of `old`.  One instruction instead of two
+// unpacks, two multiplies and a conversion; bit-identical to them for every bf16 value that the
+// scale rule allows (|x| / scale <= 448), checked exhaustively on the hardware.
+template <bool HI>
+__device__ __forceinline__ uint32_t cvt2_e4m3_scaled(uint32_t old, uint32_t pair, float scale) {
+  const s16x2 r = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(__builtin_bit_cast(s16x2, old), __builtin_bit_cast(bf16x2_t, pair),
+                                                            scale, HI);
+  return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint32_t cvt4_e4m3_scaled(uint32_t p01, uint32_t p23, float scale) {
+  return cvt2_e4m3_scaled<true>(cvt2_e4m3_scaled<false>(0u, p01, scale), p23, scale);
+}
 
+// One 128x128 tile.  FULL: the tile lies inside the tensor and every vector access is legal, so no
+// bounds are checked; for bf16 sources it also selects the packed arithmetic above.
+template <typename T, int AM, int BMODE, int BL, int BS, int PRO, bool FULL>
+__device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_colmax)[128], float* s_blk, uint8_t* s_t,
+                                                const int tc, const int tr, const int64_t g) {
+  constexpr bool PK = FULL && std::is_same<T, bf16_tag>::value;  // packed-bf16 arithmetic
   const int t = threadIdx.x;
   const int cc = t & 15, rg = t >> 4, wave = t >> 6, lane = t & 63;
-  int64_t bid = blockIdx.x;
-  // PRO_SILU_BWD_PAIR: one workgroup produces the dgate tile and its dup twin (half / 128 column
-  // tiles further right) from one read of grad_h, gate and up
-  const int tiles_n_grid = PRO == PRO_SILU_BWD_PAIR ? p.tiles_n / 2 : p.tiles_n;
-  const int tc = (int)(bid % tiles_n_grid); bid /= tiles_n_grid;
-  const int tr = (int)(bid % p.tiles_m);
-  const int64_t g = bid / p.tiles_m;
-
   const int64_t row0 = (int64_t)tr * 128 + rg * 8;
   const int64_t col0 = (int64_t)tc * 128 + cc * 8;
   const char* xb = reinterpret_cast<const char*>(p.x) + g * p.x_stride_g * Loader<T>::kBytes;
@@ -124,10 +148,10 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   Frag<T> f;
   [[maybe_unused]] Frag<T> f_up;  // PRO_SILU_BWD_PAIR only
   if constexpr (PRO == PRO_SILU_BWD_PAIR) {
-    const bool col_ok = col0 < p.half;
+    const bool col_ok = FULL || col0 < p.half;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      if (col_ok && row0 + i < p.M) {
+      if (FULL || (col_ok && row0 + i < p.M)) {
         const int64_t r = row0 + i;
         float d[8], g[8], u[8], dg[8], du[8];
         st_bf16::load8(xb + (r * p.ldx + col0) * 2, d);
@@ -149,10 +173,10 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
     // The quantised tensor is the bf16-rounded SwiGLU output (forward: h = silu(gate) * up from
     // gate_up = x) or its gradient (backward: [dgate | dup] from grad_h = x and gate_up = x2),
     // computed here instead of being written to memory and read back.  bf16 only, 16-byte loads.
-    const bool col_ok = col0 < p.N;
+    const bool col_ok = FULL || col0 < p.N;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      if (col_ok && row0 + i < p.M) {
+      if (FULL || (col_ok && row0 + i < p.M)) {
         const int64_t r = row0 + i;
         float g[8], u[8], o[8];
         if (PRO == PRO_SILU_FWD) {
@@ -182,13 +206,13 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
         f.zero_row(i);
       }
     }
-  } else if (p.vec_in) {
-    const bool col_ok = col0 < p.N;
+  } else if (FULL || p.vec_in) {
+    const bool col_ok = FULL || col0 < p.N;
     int32_t src[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) src[i] = 0;
     if (p.row_index) {
-      if (row0 + 8 <= p.M) {  // the thread's 8 rows are consecutive: two 16-byte index loads (row0 % 8 == 0)
+      if (FULL || row0 + 8 <= p.M) {  // the thread's 8 rows are consecutive: two 16-byte index loads (row0 % 8 == 0)
         const int4 lo = *reinterpret_cast<const int4*>(p.row_index + row0);
         const int4 hi = *reinterpret_cast<const int4*>(p.row_index + row0 + 4);
         src[0] = lo.x; src[1] = lo.y; src[2] = lo.z; src[3] = lo.w; src[4] = hi.x; src[5] = hi.y; src[6] = hi.z; src[7] = hi.w;
@@ -198,11 +222,18 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
           if (row0 + i < p.M) src[i] = p.row_index[row0 + i];
       }
     }
+    if (FULL && !p.row_index) {
+      const char* base = xb + (row0 * p.ldx + col0) * Loader<T>::kBytes;
+      const int64_t pitch = p.ldx * Loader<T>::kBytes;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int64_t sr = p.row_index ? (int64_t)src[i] : row0 + i;
-      if (col_ok && row0 + i < p.M && sr >= 0) f.load_row(i, xb + (sr * p.ldx + col0) * Loader<T>::kBytes);
-      else f.zero_row(i);
+      for (int i = 0; i < 8; ++i) f.load_row(i, base + i * pitch);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int64_t sr = p.row_index ? (int64_t)src[i] : row0 + i;
+        if ((FULL || (col_ok && row0 + i < p.M)) && sr >= 0) f.load_row(i, xb + (sr * p.ldx + col0) * Loader<T>::kBytes);
+        else f.zero_row(i);
+      }
     }
   } else {
 #pragma unroll
@@ -220,12 +251,18 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   auto quantise_tile = [&](const int tc, const int64_t col0, Frag<T>& f) {
   // ---- reductions ------------------------------------------------------------------------
   float rowmax[8];
+  if constexpr (PK) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    float m = fabsf(f.get(i, 0));
+    for (int i = 0; i < 8; ++i)
+      rowmax[i] = pk_hmax_f32(pk_umax(pk_umax(pk_abs(f.w[i][0]), pk_abs(f.w[i][1])), pk_umax(pk_abs(f.w[i][2]), pk_abs(f.w[i][3]))));
+  } else {
 #pragma unroll
-    for (int j = 1; j < 8; ++j) m = fmaxf(m, fabsf(f.get(i, j)));
-    rowmax[i] = m;
+    for (int i = 0; i < 8; ++i) {
+      float m = fabsf(f.get(i, 0));
+#pragma unroll
+      for (int j = 1; j < 8; ++j) m = fmaxf(m, fabsf(f.get(i, j)));
+      rowmax[i] = m;
+    }
   }
   if (AM == A_ROW) {
 #pragma unroll
@@ -240,19 +277,26 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       f.fence_row(i);
-      float rcp;
+      float rcp, s;
       if (AM == A_ROW) {
-        const float s = fp8_scale_from_amax(rowmax[i], rcp);
-        if (cc == 0 && row0 + i < p.M) p.a_scale[(row0 + i) * nb + tc] = s;
+        s = fp8_scale_from_amax(rowmax[i], rcp);
+        if (cc == 0 && (FULL || row0 + i < p.M)) p.a_scale[(row0 + i) * nb + tc] = s;
       } else {
         rcp = blk_rcp;
+        s = blk_scale;
       }
-      const uint32_t lo = cvt4_e4m3(f.get(i, 0) * rcp, f.get(i, 1) * rcp, f.get(i, 2) * rcp, f.get(i, 3) * rcp);
-      const uint32_t hi = cvt4_e4m3(f.get(i, 4) * rcp, f.get(i, 5) * rcp, f.get(i, 6) * rcp, f.get(i, 7) * rcp);
-      if (row0 + i < p.M) {
+      uint32_t lo, hi;
+      if constexpr (PK) {
+        lo = cvt4_e4m3_scaled(f.w[i][0], f.w[i][1], s);
+        hi = cvt4_e4m3_scaled(f.w[i][2], f.w[i][3], s);
+      } else {
+        lo = cvt4_e4m3(f.get(i, 0) * rcp, f.get(i, 1) * rcp, f.get(i, 2) * rcp, f.get(i, 3) * rcp);
+        hi = cvt4_e4m3(f.get(i, 4) * rcp, f.get(i, 5) * rcp, f.get(i, 6) * rcp, f.get(i, 7) * rcp);
+      }
+      if (FULL || row0 + i < p.M) {
         uint8_t* dst = ab + (row0 + i) * p.N + col0;
-        if (p.vec_out) {
-          if (col0 < p.N) *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+        if (FULL || p.vec_out) {
+          if (FULL || col0 < p.N) *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
         } else {
 #pragma unroll
           for (int j = 0; j < 8; ++j)
@@ -272,18 +316,32 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   f.fence();
   float colmax[8];
   if (BMODE == B_COL) {
+    if constexpr (PK) {
+      // columns stay packed in pairs through the in-wave and the cross-wave reduction
+      uint32_t* s_pair = reinterpret_cast<uint32_t*>(&s_colmax[0][0]);  // [4][64] pairs
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      float m = fabsf(f.get(0, j));
+      for (int k = 0; k < 4; ++k) {
+        uint32_t m = pk_abs(f.w[0][k]);
 #pragma unroll
-      for (int i = 1; i < 8; ++i) m = fmaxf(m, fabsf(f.get(i, j)));
-      m = fmaxf(m, __shfl_xor(m, 16));
-      m = fmaxf(m, __shfl_xor(m, 32));
-      colmax[j] = m;
-    }
-    if (lane < 16) {
+        for (int i = 1; i < 8; ++i) m = pk_umax(m, pk_abs(f.w[i][k]));
+        m = pk_umax(m, (uint32_t)__shfl_xor((int)m, 16));
+        m = pk_umax(m, (uint32_t)__shfl_xor((int)m, 32));
+        if (lane < 16) s_pair[wave * 64 + cc * 4 + k] = m;
+      }
+    } else {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) s_colmax[wave][cc * 8 + j] = colmax[j];
+      for (int j = 0; j < 8; ++j) {
+        float m = fabsf(f.get(0, j));
+#pragma unroll
+        for (int i = 1; i < 8; ++i) m = fmaxf(m, fabsf(f.get(i, j)));
+        m = fmaxf(m, __shfl_xor(m, 16));
+        m = fmaxf(m, __shfl_xor(m, 32));
+        colmax[j] = m;
+      }
+      if (lane < 16) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s_colmax[wave][cc * 8 + j] = colmax[j];
+      }
     }
   }
   float blkmax = 0.f;
@@ -298,10 +356,21 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   }
   __syncthreads();
   if (BMODE == B_COL) {
+    if constexpr (PK) {
+      const uint32_t* s_pair = reinterpret_cast<const uint32_t*>(&s_colmax[0][0]);
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      colmax[j] = fmaxf(fmaxf(s_colmax[0][cc * 8 + j], s_colmax[1][cc * 8 + j]),
-                        fmaxf(s_colmax[2][cc * 8 + j], s_colmax[3][cc * 8 + j]));
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t m = pk_umax(pk_umax(s_pair[cc * 4 + k], s_pair[64 + cc * 4 + k]),
+                                   pk_umax(s_pair[128 + cc * 4 + k], s_pair[192 + cc * 4 + k]));
+        colmax[2 * k] = __uint_as_float(m << 16);
+        colmax[2 * k + 1] = __uint_as_float(m & 0xFFFF0000u);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        colmax[j] = fmaxf(fmaxf(s_colmax[0][cc * 8 + j], s_colmax[1][cc * 8 + j]),
+                          fmaxf(s_colmax[2][cc * 8 + j], s_colmax[3][cc * 8 + j]));
+    }
   }
   float blk_scale = 0.f, blk_rcp = 0.f;
   if (AM == A_BLOCK || BMODE == B_BLOCK) {
@@ -314,19 +383,19 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
 
   // ---- twin ---------------------------------------------------------------------------------
   f.fence();
-  float crcp[8];
+  float crcp[8], cs[8];
   if (BMODE == B_COL) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float s = fp8_scale_from_amax(colmax[j], crcp[j]);
-      if (rg == 0 && col0 + j < p.N) {
-        if (BS == BS_MB_N) p.b_scale[(int64_t)tr * p.N + col0 + j] = s;
-        else               p.b_scale[(col0 + j) * (int64_t)p.tiles_m + tr] = s;
+      cs[j] = fp8_scale_from_amax(colmax[j], crcp[j]);
+      if (rg == 0 && (FULL || col0 + j < p.N)) {
+        if (BS == BS_MB_N) p.b_scale[(int64_t)tr * p.N + col0 + j] = cs[j];
+        else               p.b_scale[(col0 + j) * (int64_t)p.tiles_m + tr] = cs[j];
       }
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) crcp[j] = blk_rcp;
+    for (int j = 0; j < 8; ++j) { crcp[j] = blk_rcp; cs[j] = blk_scale; }
     if (t == 0) p.b_scale[g * p.b_scale_stride_g + (int64_t)tc * p.tiles_m + tr] = blk_scale;
   }
 
@@ -337,10 +406,10 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
       f.fence_row(i);
       const uint32_t lo = cvt4_e4m3(f.get(i, 0) * crcp[0], f.get(i, 1) * crcp[1], f.get(i, 2) * crcp[2], f.get(i, 3) * crcp[3]);
       const uint32_t hi = cvt4_e4m3(f.get(i, 4) * crcp[4], f.get(i, 5) * crcp[5], f.get(i, 6) * crcp[6], f.get(i, 7) * crcp[7]);
-      if (row0 + i < p.M) {
+      if (FULL || row0 + i < p.M) {
         uint8_t* dst = bb + (row0 + i) * p.N + col0;
-        if (p.vec_out) {
-          if (col0 < p.N) *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+        if (FULL || p.vec_out) {
+          if (FULL || col0 < p.N) *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
         } else {
 #pragma unroll
           for (int j = 0; j < 8; ++j)
@@ -351,14 +420,39 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
   } else {
     // pack 8 consecutive rows of each column and stage the transposed tile in LDS:
     // s_t[n][m], 16-byte chunk index XOR-swizzled with (n >> 3) & 7.
+    if constexpr (PK) {
+      // A byte permute puts the same column of two consecutive rows into one register pair, which
+      // the scaled conversion then turns into two bytes that are already neighbours in the
+      // transposed row.
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float r = crcp[j];
-      const uint32_t lo = cvt4_e4m3(f.get(0, j) * r, f.get(1, j) * r, f.get(2, j) * r, f.get(3, j) * r);
-      const uint32_t hi = cvt4_e4m3(f.get(4, j) * r, f.get(5, j) * r, f.get(6, j) * r, f.get(7, j) * r);
-      const int n = cc * 8 + j;
-      const int chunk = (rg >> 1) ^ ((n >> 3) & 7);
-      *reinterpret_cast<uint2*>(&s_t[n * 128 + chunk * 16 + (rg & 1) * 8]) = make_uint2(lo, hi);
+      for (int k = 0; k < 4; ++k) {
+        uint32_t even[4], odd[4];  // row pairs (0,1) (2,3) (4,5) (6,7) of columns 2k and 2k+1
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          even[q] = __builtin_amdgcn_perm(f.w[2 * q + 1][k], f.w[2 * q][k], 0x05040100u);
+          odd[q] = __builtin_amdgcn_perm(f.w[2 * q + 1][k], f.w[2 * q][k], 0x07060302u);
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int j = 2 * k + h;
+          const uint32_t* pr = h ? odd : even;
+          const uint32_t lo = cvt4_e4m3_scaled(pr[0], pr[1], cs[j]);
+          const uint32_t hi = cvt4_e4m3_scaled(pr[2], pr[3], cs[j]);
+          const int n = cc * 8 + j;
+          const int chunk = (rg >> 1) ^ ((n >> 3) & 7);
+          *reinterpret_cast<uint2*>(&s_t[n * 128 + chunk * 16 + (rg & 1) * 8]) = make_uint2(lo, hi);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float r = crcp[j];
+        const uint32_t lo = cvt4_e4m3(f.get(0, j) * r, f.get(1, j) * r, f.get(2, j) * r, f.get(3, j) * r);
+        const uint32_t hi = cvt4_e4m3(f.get(4, j) * r, f.get(5, j) * r, f.get(6, j) * r, f.get(7, j) * r);
+        const int n = cc * 8 + j;
+        const int chunk = (rg >> 1) ^ ((n >> 3) & 7);
+        *reinterpret_cast<uint2*>(&s_t[n * 128 + chunk * 16 + (rg & 1) * 8]) = make_uint2(lo, hi);
+      }
     }
     __syncthreads();
     // destination of tile element (n, m): base + n * ld + m
@@ -370,13 +464,11 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
     } else {
       const int64_t row_start = (int64_t)tr * 128;
       int grp = 0;
-      int64_t gstart = 0, gend = 0;
+      int64_t gstart = 0;
       for (int q = 0; q < p.num_groups; ++q) {  // uniform scalar scan; groups are 128-aligned
         const int64_t e = p.offs[q];
         if (e <= row_start && q < p.num_groups - 1) { grp = q + 1; gstart = e; }
       }
-      gend = p.offs[grp];
-      (void)gend;
       const int64_t kg = (int64_t)p.offs[grp] - gstart;
       base = p.b_out + gstart * p.N + (int64_t)tc * 128 * kg + (row_start - gstart);
       ld = kg;
@@ -387,11 +479,11 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
       const int n = (t >> 3) + 32 * k;
       const int64_t gn = (int64_t)tc * 128 + n;
       const int64_t gm = (int64_t)tr * 128 + mc * 16;
-      if (gn >= p.N) continue;
+      if (!FULL && gn >= p.N) continue;
       const uint4 val = *reinterpret_cast<const uint4*>(&s_t[n * 128 + ((mc ^ ((n >> 3) & 7)) * 16)]);
       uint8_t* dst = base + n * ld + mc * 16;
-      if (p.vec_out_t) {
-        if (gm < p.M) *reinterpret_cast<uint4*>(dst) = val;
+      if (FULL || p.vec_out_t) {
+        if (FULL || gm < p.M) *reinterpret_cast<uint4*>(dst) = val;
       } else {
         const uint32_t w[4] = {val.x, val.y, val.z, val.w};
 #pragma unroll
@@ -406,6 +498,26 @@ __global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
     __syncthreads();  // the shared staging arrays are reused by the twin
     quantise_tile(tc + p.tiles_n / 2, col0 + p.half, f_up);
   }
+}
+
+template <typename T, int AM, int BMODE, int BL, int BS, int PRO = PRO_NONE>
+__global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
+  __shared__ float s_colmax[4][128];
+  __shared__ float s_blk[4];
+  __shared__ __attribute__((aligned(16))) uint8_t s_t[128 * 128];
+
+  int64_t bid = blockIdx.x;
+  // PRO_SILU_BWD_PAIR: one workgroup produces the dgate tile and its dup twin (half / 128 column
+  // tiles further right) from one read of grad_h, gate and up
+  const int tiles_n_grid = PRO == PRO_SILU_BWD_PAIR ? p.tiles_n / 2 : p.tiles_n;
+  const int tc = (int)(bid % tiles_n_grid); bid /= tiles_n_grid;
+  const int tr = (int)(bid % p.tiles_m);
+  const int64_t g = bid / p.tiles_m;
+  // interior tile with every vector access legal (uniform over the workgroup)
+  const int64_t n_cols = PRO == PRO_SILU_BWD_PAIR ? p.half : p.N;
+  const bool full = (int64_t)tr * 128 + 128 <= p.M && (int64_t)tc * 128 + 128 <= n_cols && p.vec_in && p.vec_out && p.vec_out_t;
+  if (full) quant_tile_body<T, AM, BMODE, BL, BS, PRO, true>(p, s_colmax, s_blk, s_t, tc, tr, g);
+  else      quant_tile_body<T, AM, BMODE, BL, BS, PRO, false>(p, s_colmax, s_blk, s_t, tc, tr, g);
 }
 
 template <int AM, int BMODE, int BL, int BS>
