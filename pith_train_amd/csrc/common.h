@@ -28,16 +28,16 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
 
-// fp32 -> bf16 round-to-nearest-even (NaN kept quiet)
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return u >> 16;
-}
+// fp32 -> bf16 round-to-nearest-even (NaN kept quiet) with the hardware conversion
+// (v_cvt_pk_bf16_f32): one instruction per pair, and bit-identical to the integer sequence
+// u += 0x7FFF + ((u >> 16) & 1); u >>= 16 for all 2^32 inputs (checked exhaustively on MI355X).
+typedef __bf16 pt_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float pt_f32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  const pt_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, pt_bf16x2));
 }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return pack_bf16x2(f, 0.f) & 0xFFFFu; }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)b);

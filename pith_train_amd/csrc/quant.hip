@@ -149,10 +149,14 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
   [[maybe_unused]] Frag<T> f_up;  // PRO_SILU_BWD_PAIR only
   if constexpr (PRO == PRO_SILU_BWD_PAIR) {
     const bool col_ok = FULL || col0 < p.half;
+    // Two rows in flight: row i + 2 is addressed through a register that an empty assembly statement
+    // ties to the packed results of row i.  Left alone, the compiler starts all eight rows at once
+    // (24 loads and their unpacked values: the whole register file, one wave per SIMD).
+    uint32_t gate[2] = {0u, 0u};  // always zero
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       if (FULL || (col_ok && row0 + i < p.M)) {
-        const int64_t r = row0 + i;
+        const int64_t r = row0 + i + gate[i & 1];
         float d[8], g[8], u[8], dg[8], du[8];
         st_bf16::load8(xb + (r * p.ldx + col0) * 2, d);
         const char* gp = (const char*)p.x2 + (r * p.ldx2 + col0) * 2;
@@ -164,6 +168,9 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
         f.w[i][2] = pack_bf16x2(dg[4], dg[5]); f.w[i][3] = pack_bf16x2(dg[6], dg[7]);
         f_up.w[i][0] = pack_bf16x2(du[0], du[1]); f_up.w[i][1] = pack_bf16x2(du[2], du[3]);
         f_up.w[i][2] = pack_bf16x2(du[4], du[5]); f_up.w[i][3] = pack_bf16x2(du[6], du[7]);
+        f.fence_row(i);
+        f_up.fence_row(i);
+        asm volatile("" : "+v"(gate[i & 1]) : "v"(f.w[i][3]), "v"(f_up.w[i][3]));
       } else {
         f.zero_row(i);
         f_up.zero_row(i);
@@ -500,8 +507,12 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
   }
 }
 
+// Register budget: the kernel is bound by memory latency, so resident waves matter more than
+// keeping every load of a tile in flight at once (which is what the compiler does when it is given
+// the whole register file: 256 registers and one wave per SIMD for the paired SwiGLU backward).
 template <typename T, int AM, int BMODE, int BL, int BS, int PRO = PRO_NONE>
-__global__ __launch_bounds__(256) void quant_tile_kernel(QuantArgs p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PRO == PRO_SILU_BWD_PAIR ? 3 : (BL == BL_ROWMAJOR ? 5 : 6))))
+void quant_tile_kernel(QuantArgs p) {
   __shared__ float s_colmax[4][128];
   __shared__ float s_blk[4];
   __shared__ __attribute__((aligned(16))) uint8_t s_t[128 * 128];
