@@ -154,14 +154,37 @@ class GemmTimer:
             d[1] += 1
         return {k: {"ms_total": v[0], "launches": v[1]} for k, v in out.items()}
 
-    def by_shape(self, steps):
-        """Average duration in microseconds of one launch per (entry point, M x N x K) of a step."""
+    def by_shape(self, steps, groups, routed_rows):
+        """Per (entry point, M x N x K) of a step: average duration of one launch, and the time the
+        same launch needs at the MFMA peak (algorithmic FLOPs, padding rows not counted) and at the
+        HBM peak (algorithmic bytes: both FP8 operands and their scales read once, the result
+        written once)."""
         out = {}
         for name, a, b, shape in self.records:
-            d = out.setdefault(f"{name.replace('pt_gemm_', '')} {shape}", [0.0, 0])
+            d = out.setdefault((name, shape), [0.0, 0])
             d[0] += a.elapsed_time(b)
             d[1] += 1
-        return {k: {"us": round(v[0] / v[1] * 1e3, 1), "launches_per_step": v[1] / max(steps, 1)} for k, v in out.items()}
+        rep = {}
+        for (name, shape), (ms, n) in out.items():
+            m, nn, k = (int(v) for v in shape.split("x"))
+            if name == "pt_gemm_nt_dense":
+                flop = 2.0 * m * nn * k
+                byts = m * k * (1 + 4 / 128) + nn * k * (1 + 4 / 16384) + 2.0 * m * nn
+            else:
+                real = min(m, routed_rows)  # rows that carry tokens (the rest is per-group padding)
+                flop = 2.0 * real * nn * k
+                if name == "pt_gemm_k_grouped_wgrad":  # dW[g] = dY_g^T X_g: both twins read, [G,N,K] written
+                    byts = m * (nn + k) * (1 + 4 / 128) + 2.0 * groups * nn * k
+                else:
+                    out_rows = real if name.endswith("_scatter") else m
+                    byts = m * k * (1 + 4 / 128) + groups * nn * k * (1 + 4 / 16384) + 2.0 * out_rows * nn
+            us = ms / n * 1e3
+            rep[f"{name.replace('pt_gemm_', '')} {shape}"] = {
+                "us": round(us, 1), "launches_per_step": n / max(steps, 1),
+                "mfma_floor_us": round(flop / (FP8_DENSE_PEAK_TFLOPS * 1e12) * 1e6, 1),
+                "hbm_floor_us": round(byts / (HBM_PEAK_GBS * 1e9) * 1e6, 1),
+            }
+        return rep
 
 
 def hbm_kernel_report(H, I, E, rows, eidx):
@@ -357,6 +380,8 @@ def main():
     gemm_ms = sum(v["ms_total"] for v in gs.values())
     gemm_launches = sum(v["launches"] for v in gs.values())
     achieved = flops * args.steps / (gemm_ms * 1e-3) / 1e12 if gemm_ms > 0 else 0.0
+    per_shape = timer.by_shape(args.steps, E, rows)
+    floor_ms = sum(max(v["mfma_floor_us"], v["hbm_floor_us"]) * v["launches_per_step"] for v in per_shape.values()) / 1e3
 
     extra = {}
     if not args.no_cached_weights:
@@ -418,7 +443,11 @@ def main():
             "launches_per_step": gemm_launches / max(args.steps, 1),
             "gemm_ms_per_step": gemm_ms / max(args.steps, 1),
             "per_entry_point_ms_per_step": {k2: v["ms_total"] / args.steps for k2, v in gs.items()},
-            "per_shape": timer.by_shape(args.steps),
+            "per_shape": per_shape,
+            # every launch priced at the better of the two peaks: what the step's GEMMs would take on
+            # a machine that reaches 5 PFLOP/s and 8 TB/s at once
+            "floor_ms_per_step": floor_ms,
+            "frac_of_floor": floor_ms / (gemm_ms / max(args.steps, 1)) if gemm_ms > 0 else 0.0,
         },
         **extra,
     }

@@ -26,29 +26,6 @@
 
 namespace pt {
 
-// Scaled MFMA whose scale bytes are byte `ia` of sa and byte `ib` of sb (byte index = op_sel bit +
-// 2 * op_sel_hi bit, one pair per operand).  Issued as volatile inline assembly with a memory
-// clobber: the compiler keeps such statements, and every memory operation between them, in source
-// order, which is what pins the interleaving of MFMAs, LDS reads and direct-to-LDS loads in the
-// main loop.  The accumulator lives in the accumulation registers ("a" constraint).
-__device__ __forceinline__ void mfma_sel(const v8i& a, const v8i& b, v16f& c, int ia, int sa, int ib, int sb) {
-#define PT_MFMA(IA, IB, S0, S1, H0, H1)                                                                         \
-  case IA * 4 + IB:                                                                                             \
-    asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[" #S0 "," #S1 ",0] op_sel_hi:[" #H0 \
-                 "," #H1 ",0]"                                                                                  \
-                 : "+a"(c)                                                                                      \
-                 : "v"(a), "v"(b), "v"(sa), "v"(sb)                                                             \
-                 : "memory");                                                                                   \
-    break;
-  switch (ia * 4 + ib) {
-    PT_MFMA(0, 0, 0, 0, 0, 0) PT_MFMA(0, 1, 0, 1, 0, 0) PT_MFMA(0, 2, 0, 0, 0, 1) PT_MFMA(0, 3, 0, 1, 0, 1)
-    PT_MFMA(1, 0, 1, 0, 0, 0) PT_MFMA(1, 1, 1, 1, 0, 0) PT_MFMA(1, 2, 1, 0, 0, 1) PT_MFMA(1, 3, 1, 1, 0, 1)
-    PT_MFMA(2, 0, 0, 0, 1, 0) PT_MFMA(2, 1, 0, 1, 1, 0) PT_MFMA(2, 2, 0, 0, 1, 1) PT_MFMA(2, 3, 0, 1, 1, 1)
-    PT_MFMA(3, 0, 1, 0, 1, 0) PT_MFMA(3, 1, 1, 1, 1, 0) PT_MFMA(3, 2, 1, 0, 1, 1) PT_MFMA(3, 3, 1, 1, 1, 1)
-  }
-#undef PT_MFMA
-}
-
 template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC>
 __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_pipelined_kernel(GemmArgs p) {
   constexpr int NW = WGM * WGN;
