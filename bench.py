@@ -173,11 +173,12 @@ class GemmTimer:
             else:
                 real = min(m, routed_rows)  # rows that carry tokens (the rest is per-group padding)
                 flop = 2.0 * real * nn * k
+                # (m may be the buffers' capacity rather than the padded row count, which then only
+                # the device knows: the floor counts the rows that carry tokens)
                 if name == "pt_gemm_k_grouped_wgrad":  # dW[g] = dY_g^T X_g: both twins read, [G,N,K] written
-                    byts = m * (nn + k) * (1 + 4 / 128) + 2.0 * groups * nn * k
+                    byts = real * (nn + k) * (1 + 4 / 128) + 2.0 * groups * nn * k
                 else:
-                    out_rows = real if name.endswith("_scatter") else m
-                    byts = m * k * (1 + 4 / 128) + groups * nn * k * (1 + 4 / 16384) + 2.0 * out_rows * nn
+                    byts = real * k * (1 + 4 / 128) + groups * nn * k * (1 + 4 / 16384) + 2.0 * real * nn
             us = ms / n * 1e3
             rep[f"{name.replace('pt_gemm_', '')} {shape}"] = {
                 "us": round(us, 1), "launches_per_step": n / max(steps, 1),

@@ -42,8 +42,11 @@ enum {
 };
 
 /* 1x128 rowwise + 128-row colwise from one read.  M % 128 == 0 (deepgemm_quantize.py:219).
- * offs/num_groups are read only for PT_CH_KMAJOR (int32 inclusive row offsets, multiples of 128,
- * offs[num_groups-1] == M). */
+ * offs/num_groups (int32 inclusive row offsets, multiples of 128) give the PT_CH_KMAJOR layout its
+ * groups.  For every layout, when offs is given, offs[num_groups-1] is the number of rows that
+ * are quantised: M may then be an upper bound known on the host (buffers sized for the largest
+ * row count a routing can produce) while the real count stays in device memory, and row tiles at
+ * or past it are left untouched.  Without offs all M rows are quantised. */
 int pt_quant_rowwise_colwise(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
                              void* tok_fp8, float* tok_scale, void* ch_fp8, float* ch_scale,
                              int ch_layout, const int32_t* offs, int32_t num_groups,
@@ -63,17 +66,21 @@ int pt_quant_rowwise_colwise_rows(const void* x, int dtype, int64_t M, int64_t N
  * with gate = gate_up[:, :half], up = gate_up[:, half:], quantised as pt_quant_rowwise_colwise
  * with the PT_CH_TRANSPOSED twin: tok_fp8[M,half], tok_scale[M,ceil(half/128)], ch_t_fp8[half,M],
  * ch_scale[M/128,half].  Same bits as silu_mul (silu_mul.py:28-49) followed by
- * fp8cast_rowwise_colwise (deepgemm_quantize.py:204-259); h itself is never written. */
+ * fp8cast_rowwise_colwise (deepgemm_quantize.py:204-259); h itself is never written.
+ * valid_rows (optional, device): *valid_rows rows are processed, the row tiles past them are left
+ * untouched (M is then the host-side upper bound the buffers are sized for). */
 int pt_silu_mul_quant_rowwise_colwise(const void* gate_up, int64_t M, int64_t half,
                                       int64_t ld_gate_up, void* tok_fp8, float* tok_scale,
-                                      void* ch_t_fp8, float* ch_scale, pt_stream_t stream);
+                                      void* ch_t_fp8, float* ch_scale, const int32_t* valid_rows,
+                                      pt_stream_t stream);
 /* Backward twin: [dgate | dup] = silu_mul backward (silu_mul.py:52-87) of grad_h[M,half] at the
  * saved gate_up[M,2*half], rounded to bf16 and quantised to tok_fp8[M,2*half],
  * tok_scale[M,ceil(2*half/128)], ch_t_fp8[2*half,M], ch_scale[M/128,2*half]. */
 int pt_silu_mul_bwd_quant_rowwise_colwise(const void* grad_h, int64_t ld_grad_h,
                                           const void* gate_up, int64_t ld_gate_up, int64_t M,
                                           int64_t half, void* tok_fp8, float* tok_scale,
-                                          void* ch_t_fp8, float* ch_scale, pt_stream_t stream);
+                                          void* ch_t_fp8, float* ch_scale, const int32_t* valid_rows,
+                                          pt_stream_t stream);
 
 /* rowwise(x) + rowwise(x^T): t_fp8[N,M], t_scale[N,ceil(M/128)].
  * fp8cast_rowwise_transpose, deepgemm_quantize.py:429-482 */

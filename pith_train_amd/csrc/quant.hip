@@ -33,6 +33,7 @@ struct QuantArgs {
   const int32_t* row_index;  // optional [M]: source row of output row r (negative: a zero row); null = identity
   const void* x2; int64_t ldx2;  // fused SwiGLU backward: the saved gate_up [M, 2*half]
   int64_t half;                  // fused SwiGLU: width of one half of gate_up
+  const int32_t* row_limit;      // optional device scalar: row tiles at or past *row_limit are skipped (nothing written)
 };
 
 template <typename T> struct Loader;
@@ -524,6 +525,9 @@ void quant_tile_kernel(QuantArgs p) {
   const int tc = (int)(bid % tiles_n_grid); bid /= tiles_n_grid;
   const int tr = (int)(bid % p.tiles_m);
   const int64_t g = bid / p.tiles_m;
+  // The caller may size the tensors for the largest row count a routing can produce and tell the
+  // real one through device memory (no host round trip): tiles past it have nothing to do.
+  if (p.row_limit && (int64_t)tr * 128 >= *p.row_limit) return;
   // interior tile with every vector access legal (uniform over the workgroup)
   const int64_t n_cols = PRO == PRO_SILU_BWD_PAIR ? p.half : p.N;
   const bool full = (int64_t)tr * 128 + 128 <= p.M && (int64_t)tc * 128 + 128 <= n_cols && p.vec_in && p.vec_out && p.vec_out_t;
@@ -550,6 +554,7 @@ static void fill_common(QuantArgs& a, const void* x, int dtype, int64_t M, int64
   a.a_stride_g = 0; a.a_scale_stride_g = 0; a.b_stride_g = 0; a.b_scale_stride_g = 0;
   a.tiles_m = (int32_t)cdiv(M, 128); a.tiles_n = (int32_t)cdiv(N, 128);
   a.offs = nullptr; a.num_groups = 0; a.row_index = nullptr; a.x2 = nullptr; a.ldx2 = 0; a.half = 0;
+  a.row_limit = nullptr;
   const int eb = dtype == PT_F32 ? 4 : 2;
   a.vec_in = (N % 8 == 0) && ((ldx * eb) % 16 == 0) && (((uintptr_t)x) % 16 == 0);
   a.vec_out = (N % 8 == 0);
@@ -592,6 +597,7 @@ static int quant_rowwise_colwise_impl(const void* x, int dtype, int64_t M, int64
   fill_common(a, x, dtype, M, N, ldx);
   a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)ch_fp8; a.b_scale = ch_scale;
   a.row_index = row_index;
+  if (offs && num_groups > 0) a.row_limit = offs + (num_groups - 1);
   hipStream_t s = (hipStream_t)stream;
   switch (ch_layout) {
     case PT_CH_ROWMAJOR:   return launch_quant<A_ROW, B_COL, BL_ROWMAJOR, BS_MB_N>(a, dtype, 1, s);
@@ -662,7 +668,7 @@ static int launch_silu_quant(const QuantArgs& a, hipStream_t stream) {
 
 extern "C" int pt_silu_mul_quant_rowwise_colwise(const void* gate_up, int64_t M, int64_t half, int64_t ld_gate_up,
                                                  void* tok_fp8, float* tok_scale, void* ch_t_fp8, float* ch_scale,
-                                                 pt_stream_t stream) {
+                                                 const int32_t* valid_rows, pt_stream_t stream) {
   PT_REQUIRE(M >= 0 && half >= 0 && M % 128 == 0 && ld_gate_up >= 2 * half, "silu_mul_quant: bad shape");
   if (M == 0 || half == 0) return PT_OK;
   PT_REQUIRE(gate_up && tok_fp8 && tok_scale && ch_t_fp8 && ch_scale, "silu_mul_quant: null pointer");
@@ -670,14 +676,15 @@ extern "C" int pt_silu_mul_quant_rowwise_colwise(const void* gate_up, int64_t M,
              "silu_mul_quant: the half width and the row stride must be multiples of 8 elements, the pointer 16-byte aligned");
   QuantArgs a;
   fill_common(a, gate_up, PT_BF16, M, half, ld_gate_up);
-  a.half = half;
+  a.half = half; a.row_limit = valid_rows;
   a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)ch_t_fp8; a.b_scale = ch_scale;
   return launch_silu_quant<PRO_SILU_FWD>(a, (hipStream_t)stream);
 }
 
 extern "C" int pt_silu_mul_bwd_quant_rowwise_colwise(const void* grad_h, int64_t ld_grad_h, const void* gate_up,
                                                      int64_t ld_gate_up, int64_t M, int64_t half, void* tok_fp8,
-                                                     float* tok_scale, void* ch_t_fp8, float* ch_scale, pt_stream_t stream) {
+                                                     float* tok_scale, void* ch_t_fp8, float* ch_scale,
+                                                     const int32_t* valid_rows, pt_stream_t stream) {
   PT_REQUIRE(M >= 0 && half >= 0 && M % 128 == 0 && ld_gate_up >= 2 * half && ld_grad_h >= half, "silu_mul_bwd_quant: bad shape");
   if (M == 0 || half == 0) return PT_OK;
   PT_REQUIRE(grad_h && gate_up && tok_fp8 && tok_scale && ch_t_fp8 && ch_scale, "silu_mul_bwd_quant: null pointer");
@@ -686,7 +693,7 @@ extern "C" int pt_silu_mul_bwd_quant_rowwise_colwise(const void* grad_h, int64_t
              "silu_mul_bwd_quant: widths and row strides must be multiples of 8 elements, pointers 16-byte aligned");
   QuantArgs a;
   fill_common(a, grad_h, PT_BF16, M, 2 * half, ld_grad_h);
-  a.half = half; a.x2 = gate_up; a.ldx2 = ld_gate_up;
+  a.half = half; a.x2 = gate_up; a.ldx2 = ld_gate_up; a.row_limit = valid_rows;
   a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)ch_t_fp8; a.b_scale = ch_scale;
   // with whole 128-column tiles per half, each workgroup makes a dgate tile and its dup twin
   if (half % 128 == 0) return launch_silu_quant<PRO_SILU_BWD_PAIR>(a, (hipStream_t)stream);

@@ -153,14 +153,17 @@ class GptOssExperts(nn.Module):
 
 
 def forward_stage3(experts: nn.Module, gathered_tokens, expert_idxs, experts_per_rank: int, expand_idx=None,
-                   fuse_expand: bool = True, fuse_permute: bool = True):
+                   fuse_expand: bool = True, fuse_permute: bool = True, host_sizes: bool = False):
     """Expert compute between the dispatch and combine all-to-alls.
 
     With ``fuse_permute`` (FP8 Qwen3 / DeepSeek / Qwen3.5 experts, no ``expand_idx``) the permuted
     copy of the tokens, its inverse gather and their two backward passes are never materialised:
     only the index half of the scatter runs, the first quantisation reads rows through the
     source map and the last GEMM of forward and of backward stores rows through it.  The result
-    is bit-identical to the unfused composition.
+    is bit-identical to the unfused composition.  Unless ``host_sizes`` is set, this path also
+    drops the scatter's device-to-host copy of the group sizes (token_scatter.py:230-243 waits for
+    the GPU there on every call): buffers are sized for the largest padded row count the routing
+    could produce and every kernel reads the real count from ``grouped_mm_offs``.
 
     ``expand_idx`` (EP > 1) re-expands the deduplicated received rows to one row per routed
     (token, expert) pair.  With ``fuse_expand`` that gather is folded into the scatter's row copy
@@ -171,8 +174,10 @@ def forward_stage3(experts: nn.Module, gathered_tokens, expert_idxs, experts_per
             and isinstance(experts, (Qwen3MoeExperts, Qwen35MoeExperts))
             and isinstance(experts.down_proj, FP8GroupedLinear)
             and experts.down_proj.out_features % 8 == 0 and experts.down_proj.in_features % 8 == 0):
+        fused_node = isinstance(experts, Qwen35MoeExperts) and fused_experts.supported(
+            gathered_tokens, experts.gate_up_proj.weight, experts.down_proj.weight)
         _, grouped_mm_offs, ks, ks_tensor, src_of = group_rows_with_sizes(
-            expert_idxs, experts_per_rank, device=gathered_tokens.device)
+            expert_idxs, experts_per_rank, device=gathered_tokens.device, host_sizes=host_sizes or not fused_node)
         return experts(gathered_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, row_map=src_of)
     if (fuse_permute and expand_idx is None and training.fp8 and expert_idxs.shape[0] > 0
             and isinstance(experts, GptOssExperts)):

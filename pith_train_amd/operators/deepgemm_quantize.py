@@ -73,9 +73,11 @@ def fp8cast_rowwise_colwise(x: torch.Tensor):
     return _rowwise_colwise(x, _lib.PT_CH_ROWMAJOR, None)
 
 
-def fp8cast_rowwise_colwise_t_rows(x: torch.Tensor, row_index: torch.Tensor):
+def fp8cast_rowwise_colwise_t_rows(x: torch.Tensor, row_index: torch.Tensor, grouped_mm_offs: torch.Tensor | None = None):
     """:func:`fp8cast_rowwise_colwise_t` of ``x[row_index]`` (rows with a negative index are zero)
-    without materialising the gathered tensor.  ``row_index`` is int32 ``[M]``, ``M % 128 == 0``."""
+    without materialising the gathered tensor.  ``row_index`` is int32 ``[M]``, ``M % 128 == 0``.
+    With ``grouped_mm_offs`` (int32, inclusive) only the rows below its last entry are written:
+    ``M`` may then be an upper bound of the row count that is only known on the device."""
     assert x.ndim == 2 and row_index.ndim == 1 and row_index.dtype == torch.int32
     assert row_index.shape[0] % 128 == 0, f"row count {row_index.shape[0]} must be a multiple of 128"
     x = _prep2d(x)
@@ -92,7 +94,8 @@ def fp8cast_rowwise_colwise_t_rows(x: torch.Tensor, row_index: torch.Tensor):
         _lib.call(
             "pt_quant_rowwise_colwise_rows", x.data_ptr(), _lib.dtype_code(x.dtype), M, N, ld,
             row_index.data_ptr(), out_tok.data_ptr(), scale_tok.data_ptr(), out_ch.data_ptr(),
-            scale_ch.data_ptr(), _lib.PT_CH_TRANSPOSED, None, 0, _lib.stream_ptr(dev),
+            scale_ch.data_ptr(), _lib.PT_CH_TRANSPOSED, _lib.ptr(grouped_mm_offs),
+            0 if grouped_mm_offs is None else grouped_mm_offs.numel(), _lib.stream_ptr(dev),
         )  # fmt: skip
     return out_tok, scale_tok, out_ch, scale_ch
 

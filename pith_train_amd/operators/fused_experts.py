@@ -22,8 +22,15 @@ def _cdiv(a: int, b: int) -> int:
     return (a + b - 1) // b
 
 
-def silu_mul_quant(gate_up: torch.Tensor):
-    """``fp8cast_rowwise_colwise_t(silu_mul(gate_up[:, :I], gate_up[:, I:]))`` in one pass."""
+def _last(offs):
+    """Device pointer to the last entry of the inclusive group offsets (= the number of grouped rows)."""
+    return None if offs is None or offs.numel() == 0 else offs.data_ptr() + 4 * (offs.numel() - 1)
+
+
+def silu_mul_quant(gate_up: torch.Tensor, grouped_mm_offs: torch.Tensor | None = None):
+    """``fp8cast_rowwise_colwise_t(silu_mul(gate_up[:, :I], gate_up[:, I:]))`` in one pass.  With
+    ``grouped_mm_offs`` only the rows below its last entry are processed (the tensors may be sized
+    for more rows than the routing produced)."""
     M, two_i = gate_up.shape
     half = two_i // 2
     dev = gate_up.device
@@ -33,13 +40,15 @@ def silu_mul_quant(gate_up: torch.Tensor):
     ch_s = torch.empty((M // 128, half), dtype=torch.float32, device=dev)
     _lib.call(
         "pt_silu_mul_quant_rowwise_colwise", gate_up.data_ptr(), M, half, gate_up.stride(0),
-        tok.data_ptr(), tok_s.data_ptr(), ch_t.data_ptr(), ch_s.data_ptr(), _lib.stream_ptr(dev),
+        tok.data_ptr(), tok_s.data_ptr(), ch_t.data_ptr(), ch_s.data_ptr(), _last(grouped_mm_offs),
+        _lib.stream_ptr(dev),
     )  # fmt: skip
     return tok, tok_s, ch_t, ch_s
 
 
-def silu_mul_bwd_quant(grad_h: torch.Tensor, gate_up: torch.Tensor):
-    """``fp8cast_rowwise_colwise_t`` of the SwiGLU gradient ``[dgate | dup]`` in one pass."""
+def silu_mul_bwd_quant(grad_h: torch.Tensor, gate_up: torch.Tensor, grouped_mm_offs: torch.Tensor | None = None):
+    """``fp8cast_rowwise_colwise_t`` of the SwiGLU gradient ``[dgate | dup]`` in one pass (rows
+    limited as in :func:`silu_mul_quant`)."""
     M, two_i = gate_up.shape
     half = two_i // 2
     dev = gate_up.device
@@ -50,7 +59,7 @@ def silu_mul_bwd_quant(grad_h: torch.Tensor, gate_up: torch.Tensor):
     _lib.call(
         "pt_silu_mul_bwd_quant_rowwise_colwise", grad_h.data_ptr(), grad_h.stride(0), gate_up.data_ptr(),
         gate_up.stride(0), M, half, tok.data_ptr(), tok_s.data_ptr(), ch_t.data_ptr(), ch_s.data_ptr(),
-        _lib.stream_ptr(dev),
+        _last(grouped_mm_offs), _lib.stream_ptr(dev),
     )  # fmt: skip
     return tok, tok_s, ch_t, ch_s
 
@@ -66,7 +75,9 @@ class FP8SwiGLUExpertsFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, w_gate_up, w_down, grouped_mm_offs, ks, ks_tensor, q_gate_up, q_down, row_map=None):
         """``x`` is ``[M, K]`` grouped rows, or with ``row_map`` (int32 ``[M]``) the un-permuted
-        ``[m, K]`` tokens; the result has the same row layout as ``x``."""
+        ``[m, K]`` tokens; the result has the same row layout as ``x``.  ``row_map`` may be longer
+        than the grouped rows (its tail negative): every kernel takes the real row count from
+        ``grouped_mm_offs`` on the device, so no host-side size is needed (``ks`` may be None)."""
         _lib.require_cuda(x)
         gu_fp8, gu_scale, gu_t_fp8, gu_t_scale = q_gate_up
         dn_fp8, dn_scale, dn_t_fp8, dn_t_scale = q_down
@@ -74,14 +85,14 @@ class FP8SwiGLUExpertsFunc(torch.autograd.Function):
         H = w_down.shape[1]
         if row_map is not None:
             M = row_map.shape[0]
-            x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, row_map)
+            x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, row_map, grouped_mm_offs)
         else:
             M = x.shape[0]
             x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t(x)
         gate_up = torch.empty((M, two_i), device=x.device, dtype=x.dtype)
         m_grouped_fp8_gemm_nt((x_fp8, x_s), (gu_fp8, gu_scale), gate_up, grouped_mm_offs)
         del x_fp8, x_s
-        h_fp8, h_s, h_ch_t, h_ch_s = silu_mul_quant(gate_up)
+        h_fp8, h_s, h_ch_t, h_ch_s = silu_mul_quant(gate_up, grouped_mm_offs if row_map is not None else None)
         out = torch.empty((x.shape[0], H), device=x.device, dtype=x.dtype)
         m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, row_map)
         ctx.save_for_backward(gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, grouped_mm_offs, x_ch_t, x_ch_s,
@@ -100,14 +111,14 @@ class FP8SwiGLUExpertsFunc(torch.autograd.Function):
         K = w_gate_up.shape[2]
         grad_out = grad_out.contiguous()
         if row_map is not None:
-            dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t_rows(grad_out, row_map)
+            dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t_rows(grad_out, row_map, offs)
         else:
             dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t(grad_out)
         grad_h = torch.empty((M, half), device=grad_out.device, dtype=grad_out.dtype)
         m_grouped_fp8_gemm_nt((dy_fp8, dy_s), (dn_t_fp8, dn_t_scale), grad_h, offs)
         schedule_wgrad(w_down, (dy_ch_t, dy_ch_s), (h_ch_t, h_ch_s), offs)
         del dy_fp8, dy_s
-        dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s = silu_mul_bwd_quant(grad_h, gate_up)
+        dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s = silu_mul_bwd_quant(grad_h, gate_up, offs if row_map is not None else None)
         grad_x = torch.empty((rows_x, K), device=grad_out.device, dtype=grad_out.dtype)
         m_grouped_fp8_gemm_nt((dgu_fp8, dgu_s), (gu_t_fp8, gu_t_scale), grad_x, offs, row_map)
         schedule_wgrad(w_gate_up, (dgu_ch_t, dgu_ch_s), (x_ch_t, x_ch_s), offs)

@@ -52,16 +52,34 @@ def group_rows(expert_idxs: torch.Tensor, num_groups: int, padding_alignment: in
     return reverse, offs, ks_tensor, src_of
 
 
-def group_rows_with_sizes(expert_idxs: torch.Tensor, num_groups: int, padding_alignment: int = 128, device=None):
+def group_rows_with_sizes(expert_idxs: torch.Tensor, num_groups: int, padding_alignment: int = 128, device=None,
+                          host_sizes: bool = True):
     """The index half of :func:`scatter_for_grouped_gemm` on its own: returns ``(reverse i64[m],
     grouped_mm_offs i32[G], ks list[int], ks_tensor i32[G], src_of i32[sum(ks)])`` where
-    ``src_of[r]`` is the source row of grouped row r (-1 for a padding row).  No rows are moved."""
+    ``src_of[r]`` is the source row of grouped row r (-1 for a padding row).  No rows are moved.
+
+    ``host_sizes=False`` skips the device-to-host copy of the group sizes and the stream
+    synchronisation it needs: ``ks`` is None and ``src_of`` keeps its full capacity (the largest
+    padded row count ``m`` rows in ``num_groups`` groups can give, -1 past the real rows).  Callers
+    that size their buffers by ``src_of`` and take the real row count from ``grouped_mm_offs`` on
+    the device (the fused expert path) then never wait for the GPU."""
     _lib.require_cuda(expert_idxs)
     expert_idxs = expert_idxs.contiguous()
     assert expert_idxs.dtype == torch.int64, "expert_idxs must be int64"
     m = expert_idxs.shape[0]
     dev = expert_idxs.device
     max_m_padded = m + num_groups * (padding_alignment - 1)
+    if not host_sizes:
+        # Capacity = the largest padded row count, as an odd multiple of 128.  The colwise twins
+        # are [N, capacity] matrices read along rows at this pitch: with a large power of two in
+        # it, consecutive rows fall onto a few memory channels (measured: 81920 = 5 * 2**14 makes
+        # the weight-gradient GEMM 25 % slower than 74112 = 579 * 128).
+        cap = -(-max_m_padded // 128) * 128
+        if (cap // 128) % 2 == 0:
+            cap += 128
+        alloc = -(-cap // _GEMM_ALLOC_ALIGNMENT) * _GEMM_ALLOC_ALIGNMENT
+        reverse, offs, ks_tensor, src_of = group_rows(expert_idxs, num_groups, padding_alignment, alloc)
+        return reverse, offs, None, ks_tensor, src_of[:cap]
     max_m_padded = -(-max_m_padded // _GEMM_ALLOC_ALIGNMENT) * _GEMM_ALLOC_ALIGNMENT
     reverse, offs, ks_tensor, src_of = group_rows(expert_idxs, num_groups, padding_alignment, max_m_padded)
     ks_cpu = get_pinned_buffer("ks", num_groups, torch.int32)
