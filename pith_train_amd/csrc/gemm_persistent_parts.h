@@ -86,70 +86,57 @@ __device__ __forceinline__ void store_pairs_bf16(const v16f& a, __amdgpu_buffer_
     __builtin_amdgcn_raw_buffer_store_b32((int)w, out, voff, s, 0);
   }
 }
-// bf16 through a per-wave LDS staging tile (32 rows x 64 B): the accumulator layout (a lane owns
-// one column) is turned into rows, so that every lane stores 16 contiguous bytes and one store
-// instruction covers 16 rows x 64 B.  The memory pipeline spends the same time on a 4-byte and a
-// 16-byte store instruction, so this is a quarter of the store issue time of store_pairs_bf16.
-// Only this wave touches its staging tile, so a counter wait between the phases is enough.
-// voff: lane's byte offset (row lane/4, 16-byte chunk lane%4) or kOob; soff: tile row 0, column 0.
-__device__ __forceinline__ void store_staged_bf16(const v16f& a, __amdgpu_buffer_rsrc_t out, uint8_t* stg, uint32_t voff,
-                                                  uint32_t soff, uint32_t pitch, bool accumulate, int lane) {
+// bf16 through a per-wave LDS staging tile: the accumulator layout (a lane owns one column) is
+// turned into rows so that every lane stores 16 contiguous bytes.  Two horizontally adjacent
+// 32x32 blocks (64 columns: one 128-byte line per row) go through the 2 KiB tile 16 rows at a
+// time, and each store instruction then writes 8 whole 128-byte lines.  (Half lines - one block,
+// 16 rows x 64 B per instruction - cost a tenth of the dense and a quarter of the weight-gradient
+// GEMM's time in the write path; the memory pipeline spends the same time on a 4-byte and on a
+// 16-byte store instruction, which is why the stores are wide in the first place.)  Only this wave
+// touches its staging tile, and the LDS executes one wave's operations in order, so the phases
+// need compiler fences only.
+// voff[q]: the lane's byte offset for tile rows 8q + lane/8, q = 0..3 (row start + 16-byte chunk
+// lane%8, or kOob); soff: uniform byte offset added to all of them.
+__device__ __forceinline__ void store_staged_bf16_lines(const v16f& a0, const v16f& a1, __amdgpu_buffer_rsrc_t out, uint8_t* stg,
+                                                        const uint32_t (&voff)[4], uint32_t soff, bool accumulate, int lane) {
   const bool odd = lane & 1;
-  uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 64 + ((lane & 31) >> 1) * 4;
+  uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 128 + ((lane & 31) >> 1) * 4;
+  const uint8_t* rd = stg + (lane >> 3) * 128 + (lane & 7) * 16;
   // p = (row r | row r+1) of the lane's column; the even lane of a pair takes both low halves (row r,
   // columns c and c+1), the odd lane both high halves (row r+1): one byte permute of own and neighbour
   const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
 #pragma unroll
-  for (int v = 0; v < 16; v += 2) {
-    const uint32_t pk = pack2_bf16(a[v], a[v + 1]);
-    const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, false);
-    *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = __builtin_amdgcn_perm(nb, pk, sel);
-  }
-  // the reads below alias the writes above: keep the compiler from reordering them (the LDS
-  // executes one wave's operations in order, so no counter wait is needed)
-  asm volatile("" ::: "memory");
-  const uint8_t* rd = stg + (lane >> 2) * 64 + (lane & 3) * 16;
+  for (int hf = 0; hf < 2; ++hf) {  // tile rows 0-15, then 16-31
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    v4i w = *(const v4i*)(rd + h * 1024);
-    const uint32_t s = soff + h * 16 * pitch;
-    if (accumulate) {
-      const v4i old = __builtin_amdgcn_raw_buffer_load_b128(out, voff, s, 0);
+    for (int b = 0; b < 2; ++b) {
+      const v16f& a = b ? a1 : a0;
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        w[q] = (int)pack2_bf16(bf16_lo((uint32_t)old[q]) + bf16_lo((uint32_t)w[q]), bf16_hi((uint32_t)old[q]) + bf16_hi((uint32_t)w[q]));
+      for (int v = 8 * hf; v < 8 * hf + 8; v += 2) {
+        const uint32_t pk = pack2_bf16(a[v], a[v + 1]);
+        const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, false);
+        *(uint32_t*)(wr + (8 * ((v >> 2) & 1) + (v & 3)) * 128 + b * 64) = __builtin_amdgcn_perm(nb, pk, sel);
+      }
     }
-    __builtin_amdgcn_raw_buffer_store_b128(w, out, voff, s, 0);
-    // A 16-byte store reads its data registers for a few cycles after it issues; the compiler
-    // only guards that window for stores without a scalar offset, so hold the registers here.
-    asm volatile("s_nop 4" ::"v"(w) : "memory");
+    asm volatile("" ::: "memory");  // the reads below alias the writes above
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      v4i w = *(const v4i*)(rd + h * 1024);
+      const uint32_t vo = voff[2 * hf + h];
+      if (accumulate) {
+        const v4i old = __builtin_amdgcn_raw_buffer_load_b128(out, vo, soff, 0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          w[q] = (int)pack2_bf16(bf16_lo((uint32_t)old[q]) + bf16_lo((uint32_t)w[q]), bf16_hi((uint32_t)old[q]) + bf16_hi((uint32_t)w[q]));
+      }
+      __builtin_amdgcn_raw_buffer_store_b128(w, out, vo, soff, 0);
+      // A 16-byte store reads its data registers for a few cycles after it issues; the compiler
+      // only guards that window for stores without a scalar offset, so hold the registers here.
+      asm volatile("s_nop 4" ::"v"(w) : "memory");
+    }
+    asm volatile("" ::: "memory");  // the next half's writes alias these reads
   }
 }
-// As store_staged_bf16 with an arbitrary output row per lane: voff0 / voff1 are the lane's byte
-// offsets (row start + 16-byte chunk, or kOob) for tile rows lane/4 and 16 + lane/4; soff the
-// column offset in bytes.
-__device__ __forceinline__ void store_staged_bf16_rows(const v16f& a, __amdgpu_buffer_rsrc_t out, uint8_t* stg, uint32_t voff0,
-                                                       uint32_t voff1, uint32_t soff, int lane) {
-  const bool odd = lane & 1;
-  uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 64 + ((lane & 31) >> 1) * 4;
-  // p = (row r | row r+1) of the lane's column; the even lane of a pair takes both low halves (row r,
-  // columns c and c+1), the odd lane both high halves (row r+1): one byte permute of own and neighbour
-  const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
-#pragma unroll
-  for (int v = 0; v < 16; v += 2) {
-    const uint32_t pk = pack2_bf16(a[v], a[v + 1]);
-    const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, false);
-    *(uint32_t*)(wr + (8 * (v >> 2) + (v & 3)) * 64) = __builtin_amdgcn_perm(nb, pk, sel);
-  }
-  asm volatile("" ::: "memory");  // compiler fence only: same-wave LDS operations execute in order
-  const uint8_t* rd = stg + (lane >> 2) * 64 + (lane & 3) * 16;
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const v4i w = *(const v4i*)(rd + h * 1024);
-    __builtin_amdgcn_raw_buffer_store_b128(w, out, h ? voff1 : voff0, soff, 0);
-    asm volatile("s_nop 4" ::"v"(w) : "memory");  // see store_staged_bf16
-  }
-}
+
 __device__ __forceinline__ void store_single_bf16(const v16f& a, __amdgpu_buffer_rsrc_t out, uint32_t voff, uint32_t soff,
                                                   uint32_t pitch, bool accumulate) {
 #pragma unroll
@@ -289,39 +276,44 @@ __device__ __forceinline__ void store_tile(v16f (&acc)[TM][TN], const GemmArgs& 
   const __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(outp, 0, (int)((uint32_t)T.a_lim * pitch), kRsrcFlags);
   const uint32_t s_tile = (uint32_t)(T.a_row0 + wm0) * pitch + (uint32_t)(T.b_row0 + wn0) * esz;
   const int colw = T.b_row0 + wn0 + (lane & 31);
+  static_assert(TN % 2 == 0, "the wide stores take column blocks in pairs");
   if (MODE == GEMM_M_GROUPED && p.out_row_index) {
     // Result row r goes to output row out_row_index[r] (the un-permute folded into the store);
     // rows of the group's padding map to a negative index and are dropped.
     const __amdgpu_buffer_rsrc_t rs_sc = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, (int)((uint32_t)p.out_rows * pitch), kRsrcFlags);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      uint32_t vrow[2];
+      // one index load for the block row (lane -> row lane%32), handed to the lanes that store the row
+      const int r = T.a_row0 + wm0 + i * 32 + (lane & 31);
+      const int dst_of_lane = r < T.a_lim ? p.out_row_index[r] : -1;
+      uint32_t vrow[4];
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int r = T.a_row0 + wm0 + i * 32 + h * 16 + (lane >> 2);
-        const int dst = r < T.a_lim ? p.out_row_index[r] : -1;
-        vrow[h] = dst >= 0 ? (uint32_t)dst * pitch + (uint32_t)(lane & 3) * 16 : kOob;
+      for (int q = 0; q < 4; ++q) {
+        const int dst = __shfl(dst_of_lane, q * 8 + (lane >> 3));
+        vrow[q] = dst >= 0 ? (uint32_t)dst * pitch + (uint32_t)(lane & 7) * 16 : kOob;
       }
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int colc = T.b_row0 + wn0 + j * 32 + (lane & 3) * 8;
-        const bool col_ok = colc < T.b_lim;
-        if constexpr (PIN) if constexpr (PIN) asm volatile("" : "+a"(acc[i][j]));
-        store_staged_bf16_rows(acc[i][j], rs_sc, stg, col_ok ? vrow[0] : kOob, col_ok ? vrow[1] : kOob,
-                               (uint32_t)(T.b_row0 + wn0 + j * 32) * 2, lane);
+      for (int j = 0; j < TN; j += 2) {
+        const int colc = T.b_row0 + wn0 + j * 32 + (lane & 7) * 8;
+        uint32_t voff[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) voff[q] = colc < T.b_lim ? vrow[q] : kOob;
+        if constexpr (PIN) { asm volatile("" : "+a"(acc[i][j])); asm volatile("" : "+a"(acc[i][j + 1])); }
+        store_staged_bf16_lines(acc[i][j], acc[i][j + 1], rs_sc, stg, voff, (uint32_t)(T.b_row0 + wn0 + j * 32) * 2, false, lane);
       }
     }
   } else if (p.out_dtype != PT_F32 && wide_ok && (T.b_lim & 7) == 0) {
-    // rows first, then the column blocks of a row band back to back: adjacent 64-byte halves of
-    // a cache line are written by consecutive instructions
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int colc = T.b_row0 + wn0 + j * 32 + (lane & 3) * 8;
-        const uint32_t voff = colc < T.b_lim ? (uint32_t)(lane >> 2) * pitch + (uint32_t)(lane & 3) * 16 : kOob;
-        if constexpr (PIN) asm volatile("" : "+a"(acc[i][j]));
-        store_staged_bf16(acc[i][j], rs_out, stg, voff, s_tile + i * 32 * pitch + j * 64, pitch, ACC, lane);
+      for (int j = 0; j < TN; j += 2) {
+        const int colc = T.b_row0 + wn0 + j * 32 + (lane & 7) * 8;
+        uint32_t voff[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          voff[q] = colc < T.b_lim ? (uint32_t)(q * 8 + (lane >> 3)) * pitch + (uint32_t)(lane & 7) * 16 : kOob;
+        if constexpr (PIN) { asm volatile("" : "+a"(acc[i][j])); asm volatile("" : "+a"(acc[i][j + 1])); }
+        store_staged_bf16_lines(acc[i][j], acc[i][j + 1], rs_out, stg, voff, s_tile + i * 32 * pitch + j * 64, ACC, lane);
       }
   } else if (p.out_dtype != PT_F32 && pair_ok && (T.b_lim & 1) == 0) {
     const bool odd = lane & 1;
