@@ -46,6 +46,17 @@ def test_workspace_queries_need_no_gpu():
     assert _lib.query("pt_dedup_workspace_bytes", 2048, 8, 128, 8) > 0
 
 
+def test_gemm_kernel_selection_validates_names_without_a_gpu():
+    from pith_train_amd import _lib
+
+    lib = _lib.load()
+    for name in (b"auto", b"p0", b"q0", b"q1", b"t", None):
+        assert lib.pt_gemm_select_kernel(name) == 0
+    assert lib.pt_gemm_select_kernel(b"fastest") != 0
+    assert b"fastest" in lib.pt_last_error()
+    assert lib.pt_gemm_select_kernel(None) == 0
+
+
 def test_operators_refuse_cpu_tensors_loudly():
     from pith_train_amd import _lib
     from pith_train_amd.operators.deepgemm_quantize import fp8cast_rowwise_colwise

@@ -111,7 +111,10 @@ def test_stage3_permute_folded_into_quant_and_gemm_is_bit_identical(kind, E, H, 
     import functools
 
     res = []
-    for fuse, fuse_act in ((True, True), (False, False), (False, True), (True, False)):
+    # (fuse_permute, fuse_activation, host_sizes): the first is the default path, which also keeps
+    # the group sizes on the device (buffers sized for the largest padded row count)
+    for fuse, fuse_act, host_sizes in ((True, True, False), (True, True, True), (False, False, True), (False, True, True),
+                                       (True, False, True)):
         mod, params = _build(kind, E, H, I, w)
         if kind == "fused":  # the one-node SwiGLU block exists for the fused gate_up layout
             mod.forward = functools.partial(mod.forward, fuse_activation=fuse_act)
@@ -119,7 +122,7 @@ def test_stage3_permute_folded_into_quant_and_gemm_is_bit_identical(kind, E, H, 
             continue
         FP8WeightCacheControl.step()
         tok = tokens.clone().requires_grad_(True)
-        out = forward_stage3(mod, tok, ids.reshape(-1).cuda(), E, fuse_permute=fuse)
+        out = forward_stage3(mod, tok, ids.reshape(-1).cuda(), E, fuse_permute=fuse, host_sizes=host_sizes)
         out.backward(dy)
         res.append((out.detach(), tok.grad, {n: p.grad for n, p in params.items()}))
     for other in res[1:]:

@@ -141,3 +141,42 @@ def test_every_bf16_value_roundtrips_like_the_oracle():
     got = D.fp8cast_rowwise_colwise(x.cuda())
     for g, r, w in zip(got, ref, ("tok_fp8", "tok_scale", "ch_fp8", "ch_scale")):
         _eq(g, r, w)
+
+
+def test_row_limit_from_device_offsets_leaves_the_tail_untouched():
+    """With the group offsets given, only the rows below their last entry are quantised: the
+    tensors may be sized for more rows than the routing produced, without the host knowing how
+    many (no device-to-host copy).  Rows below the limit carry the same bytes as a plain call."""
+    from pith_train_amd import _lib
+    from pith_train_amd.operators import deepgemm_quantize as DQ
+    from pith_train_amd.operators import fused_experts as FE
+
+    g = torch.Generator().manual_seed(11)
+    cap, real, N = 1024, 640, 384
+    x = torch.randn((700, N), generator=g).bfloat16().cuda()
+    row_index = torch.full((cap,), -1, dtype=torch.int32)
+    row_index[:real] = torch.randint(0, 700, (real,), generator=g, dtype=torch.int32)
+    row_index[real - 40 : real] = -1  # padding rows inside the last group
+    row_index = row_index.cuda()
+    offs = torch.tensor([256, 256, real], dtype=torch.int32).cuda()
+    full = DQ.fp8cast_rowwise_colwise_t_rows(x, row_index[:real].contiguous())
+    lim = DQ.fp8cast_rowwise_colwise_t_rows(x, row_index, offs)
+    u8 = lambda t: t.view(torch.uint8)  # noqa: E731
+    assert torch.equal(u8(lim[0])[:real], u8(full[0])) and torch.equal(lim[1][:real], full[1])
+    assert torch.equal(u8(lim[2])[:, :real], u8(full[2])) and torch.equal(lim[3][: real // 128], full[3])
+
+    # the kernels must not have written past the limit: pre-filled outputs keep their sentinel
+    M, half = cap, 256
+    gate_up = torch.randn((M, 2 * half), generator=g).bfloat16().cuda()
+    gate_up[real:] = float("nan")  # rows the routing never produced hold garbage
+    ref = FE.silu_mul_quant(gate_up[:real].contiguous())
+    tok = torch.full((M, half), 0x55, dtype=torch.uint8, device="cuda")
+    tok_s = torch.full((M, half // 128), -7.0, device="cuda")
+    ch_t = torch.full((half, M), 0x55, dtype=torch.uint8, device="cuda")
+    ch_s = torch.full((M // 128, half), -7.0, device="cuda")
+    _lib.call("pt_silu_mul_quant_rowwise_colwise", gate_up.data_ptr(), M, half, gate_up.stride(0), tok.data_ptr(),
+              tok_s.data_ptr(), ch_t.data_ptr(), ch_s.data_ptr(), offs.data_ptr() + 8, _lib.stream_ptr())
+    assert torch.equal(tok[:real], u8(ref[0])) and torch.equal(tok_s[:real], ref[1])
+    assert torch.equal(ch_t[:, :real], u8(ref[2])) and torch.equal(ch_s[: real // 128], ref[3])
+    assert (tok[real:] == 0x55).all() and (tok_s[real:] == -7.0).all()
+    assert (ch_t[:, real:] == 0x55).all() and (ch_s[real // 128 :] == -7.0).all()
