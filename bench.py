@@ -188,7 +188,7 @@ class GemmTimer:
         return rep
 
 
-def hbm_kernel_report(H, I, E, rows, eidx):
+def hbm_kernel_report(H, I, E, rows, eidx, top_k=8):
     """HIP-event timings of the HBM-bound kernels of the path at this workload's shapes, called
     through the operator layer one at a time: achieved GB/s = algorithmic bytes (2 B per bf16,
     1 B per fp8 element, 4 B per 128-element scale) / time, against the 8 TB/s HBM peak."""
@@ -247,6 +247,18 @@ def hbm_kernel_report(H, I, E, rows, eidx):
         2 * rows * H * 2 + 8 * rows)
     rep("gb_* kernels (padded_index_gather backward) [rows,H]",
         timeit(lambda: TS._PaddedIndexGather.scatter_sum(src, reverse, Mp, 1024)), (rows + Mp) * H * 2 + 12 * rows)
+    # the step after the path: top-k weighted combine with the residual (forward_stage5, single rank)
+    from pith_train_amd.operators.moe_combine import moe_combine
+
+    T = rows // top_k
+    tw = torch.softmax(torch.randn((T, top_k), device="cuda", generator=g), -1)
+    res = torch.randn((T, H), device="cuda", generator=g).bfloat16()
+    srcg = src.clone().requires_grad_(True)
+    twg = tw.clone().requires_grad_(True)
+    rep("moe_combine_fwd_kernel [T,k,H]", timeit(lambda: moe_combine(srcg, twg, res)), (rows + 2 * T) * H * 2 + 4 * rows)
+    o = moe_combine(srcg, twg, res)
+    rep("moe_combine_bwd_kernel [T,k,H]", timeit(lambda: torch.autograd.grad(o, [srcg, twg], res, retain_graph=True)),
+        (2 * rows + T) * H * 2 + 8 * rows)
     return out
 
 
@@ -453,7 +465,7 @@ def main():
         **extra,
     }
     if not args.no_kernel_report:
-        result["hbm_kernels"] = hbm_kernel_report(H, I, E, rows, eidx)
+        result["hbm_kernels"] = hbm_kernel_report(H, I, E, rows, eidx, k)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(kind, H, I, E, k, T, zipf)
         if extras:

@@ -274,6 +274,26 @@ int pt_indexed_bias_add_fwd(const void* x, const void* bias, const int64_t* grou
 int pt_segment_sum(const void* x, const int32_t* offs, int32_t num_groups, void* out, int64_t M,
                    int64_t H, int dtype, int out_dtype, pt_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Top-k weighted combine with the residual: the memory-bound step that follows the expert path.
+ * forward_stage5, single-rank branch (models/qwen3_moe.py:229-237; the same expression in
+ * models/deepseek_v2.py, models/gpt_oss.py, models/qwen35_moe.py).
+ * ------------------------------------------------------------------------------------------ */
+
+/* out[t,:] = residual[t,:] + S(sum_j float(moe[t*k+j,:]) * topk_weight[t,j]): fp32 products added in
+ * the order j = 0..k-1, the sum rounded to the storage type S (dtype), the addition rounded again.
+ * moe is [T*k,H], residual and out [T,H] (leading dimensions in elements), topk_weight fp32 [T,k],
+ * 1 <= k <= 16. */
+int pt_moe_combine_fwd(const void* moe, int64_t ld_moe, const float* topk_weight,
+                       const void* residual, int64_t ld_res, void* out, int64_t ld_out, int64_t T,
+                       int32_t k, int64_t H, int dtype, pt_stream_t stream);
+/* d_moe[t*k+j,:] = S(float(grad_out[t,:]) * topk_weight[t,j]);
+ * d_weight[t,j] = sum_h grad_out[t,h] * moe[t*k+j,h] in fp32 (fixed reduction order);
+ * the gradient of the residual is grad_out itself. */
+int pt_moe_combine_bwd(const void* grad_out, int64_t ld_go, const void* moe, int64_t ld_moe,
+                       const float* topk_weight, void* d_moe, int64_t ld_dmoe, float* d_weight,
+                       int64_t T, int32_t k, int64_t H, int dtype, pt_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -84,6 +84,7 @@ struct st_bf16 {
   }
   static __device__ __forceinline__ float load1(const void* p) { return bf16_bits_to_f32(*(const uint16_t*)p); }
   static __device__ __forceinline__ void store1(void* p, float v) { *(uint16_t*)p = (uint16_t)f32_to_bf16_bits(v); }
+  static __device__ __forceinline__ float round(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }  // to the storage type and back
 };
 struct st_f16 {
   static constexpr int kBytes = 2;
@@ -101,6 +102,7 @@ struct st_f16 {
   }
   static __device__ __forceinline__ float load1(const void* p) { return f16_bits_to_f32(*(const uint16_t*)p); }
   static __device__ __forceinline__ void store1(void* p, float v) { *(uint16_t*)p = (uint16_t)f32_to_f16_bits(v); }
+  static __device__ __forceinline__ float round(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
 };
 struct st_f32 {
   static constexpr int kBytes = 4;
@@ -114,6 +116,7 @@ struct st_f32 {
   }
   static __device__ __forceinline__ float load1(const void* p) { return *(const float*)p; }
   static __device__ __forceinline__ void store1(void* p, float v) { *(float*)p = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
 };
 
 // ---- FP8 scale rule ------------------------------------------------------------------------

@@ -1,0 +1,62 @@
+"""Top-k weighted combine of the expert outputs with the residual stream.
+
+The memory-bound step right after the expert path: the single-rank branch of ``forward_stage5``
+(models/qwen3_moe.py:229-237, and the same expression in the other model files)
+
+    weighted = moe_outs.view(*topk_weight.shape, -1) * topk_weight.unsqueeze(-1)
+    return residual + weighted.sum(dim=1).to(moe_outs.dtype).view(*residual.shape)
+
+as one kernel each way instead of a product tensor, a reduction, a cast and an addition.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+
+class _MoeCombine(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, moe_outs: torch.Tensor, topk_weight: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+        _lib.require_cuda(moe_outs, topk_weight, residual)
+        assert moe_outs.ndim == 2 and topk_weight.ndim == 2, "moe_outs must be [T*k, H], topk_weight [T, k]"
+        T, k = topk_weight.shape
+        H = moe_outs.shape[1]
+        assert moe_outs.shape[0] == T * k, f"moe_outs has {moe_outs.shape[0]} rows, expected {T * k}"
+        assert residual.numel() == T * H and residual.dtype == moe_outs.dtype, "residual must be [T, H] in moe_outs' dtype"
+        assert topk_weight.dtype == torch.float32, "topk_weight must be float32 (softmax scores)"
+        moe_outs = moe_outs.contiguous()
+        res2d = residual.reshape(T, H).contiguous()
+        w = topk_weight.contiguous()
+        out = torch.empty_like(res2d)
+        _lib.call(
+            "pt_moe_combine_fwd", moe_outs.data_ptr(), H, w.data_ptr(), res2d.data_ptr(), H, out.data_ptr(), H,
+            T, k, H, _lib.dtype_code(moe_outs.dtype), _lib.stream_ptr(moe_outs.device),
+        )  # fmt: skip
+        ctx.save_for_backward(moe_outs, w)
+        ctx.res_shape = residual.shape
+        return out.view(residual.shape)
+
+    @staticmethod
+    def backward(ctx, grad_out: torch.Tensor):
+        moe_outs, w = ctx.saved_tensors
+        T, k = w.shape
+        H = moe_outs.shape[1]
+        g = grad_out.reshape(T, H).contiguous()
+        d_moe = torch.empty_like(moe_outs)
+        d_w = torch.empty_like(w)
+        _lib.call(
+            "pt_moe_combine_bwd", g.data_ptr(), H, moe_outs.data_ptr(), H, w.data_ptr(), d_moe.data_ptr(), H,
+            d_w.data_ptr(), T, k, H, _lib.dtype_code(moe_outs.dtype), _lib.stream_ptr(moe_outs.device),
+        )  # fmt: skip
+        return d_moe, d_w, grad_out
+
+
+def moe_combine(moe_outs: torch.Tensor, topk_weight: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+    """``residual + (moe_outs.view(T, k, H) * topk_weight[..., None]).sum(1).to(moe_outs.dtype)``.
+
+    ``moe_outs`` is ``[T*k, H]`` (row ``t*k + j`` = expert output of token t's j-th choice),
+    ``topk_weight`` float32 ``[T, k]``, ``residual`` any shape with ``T*H`` elements; the result
+    has the residual's shape and ``moe_outs``' dtype."""
+    return _MoeCombine.apply(moe_outs, topk_weight, residual)
