@@ -101,10 +101,7 @@ __device__ __forceinline__ void store_staged_bf16_lines(const v16f& a0, const v1
                                                         const uint32_t (&voff)[4], uint32_t soff, bool accumulate, int lane) {
   const bool odd = lane & 1;
   uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 128 + ((lane & 31) >> 1) * 4;
-  // rows 4..7 and 12..15 (written by lanes 32..63, read by lanes 32..63) keep their two 64-byte halves
-  // swapped: without that, lanes l and l + 32 of a staging write hit the same bank
-  const int flip = lane >> 5;
-  const uint8_t* rd = stg + (lane >> 3) * 128 + ((lane & 7) ^ (flip << 2)) * 16;
+  const uint8_t* rd = stg + (lane >> 3) * 128 + (lane & 7) * 16;
   // p = (row r | row r+1) of the lane's column; the even lane of a pair takes both low halves (row r,
   // columns c and c+1), the odd lane both high halves (row r+1): one byte permute of own and neighbour
   const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
@@ -117,7 +114,7 @@ __device__ __forceinline__ void store_staged_bf16_lines(const v16f& a0, const v1
       for (int v = 8 * hf; v < 8 * hf + 8; v += 2) {
         const uint32_t pk = pack2_bf16(a[v], a[v + 1]);
         const uint32_t nb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)pk, 0xB1, 0xF, 0xF, false);
-        *(uint32_t*)(wr + (8 * ((v >> 2) & 1) + (v & 3)) * 128 + (b ^ flip) * 64) = __builtin_amdgcn_perm(nb, pk, sel);
+        *(uint32_t*)(wr + (8 * ((v >> 2) & 1) + (v & 3)) * 128 + b * 64) = __builtin_amdgcn_perm(nb, pk, sel);
       }
     }
     asm volatile("" ::: "memory");  // the reads below alias the writes above
