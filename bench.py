@@ -73,12 +73,29 @@ def make_dedup_expand(rows, fraction, seed=0):
     return idx[torch.randperm(rows, generator=g)], U
 
 
+def make_routing(T, E, k, seed=0, zipf_s=None):
+    """Router logits ~N(0,1) (+ an optional Zipf(s) popularity bias: log-probabilities of a seeded
+    random ranking, centred) -> softmax -> top-k expert ids [T, k]."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn((T, E), generator=g)
+    if zipf_s is not None:
+        ranks = torch.randperm(E, generator=g).float() + 1.0
+        logp = -zipf_s * ranks.log()
+        logits = logits + (logp - logp.mean())
+    return torch.topk(logits.softmax(dim=-1), k=k, dim=-1).indices
+
+
+def gemm_flops(rows, H, I):
+    """Algorithmic GEMM FLOPs of one layer, forward + dgrad + wgrad; padding rows are not counted."""
+    return 3 * (2.0 * rows * H * 2 * I + 2.0 * rows * I * H)
+
+
 def make_inputs(kind, H, I, E, k, T, zipf, seed=0):
     import torch
 
-    from oracle import moe as OM
-
-    ids = OM.make_routing(T, E, k, seed=seed, zipf_s=zipf)
+    ids = make_routing(T, E, k, seed=seed, zipf_s=zipf)
     g = torch.Generator().manual_seed(seed)
     x = torch.randn((T, H), generator=g).bfloat16()
     dy = torch.randn((T * k, H), generator=g).bfloat16()
@@ -319,7 +336,6 @@ def main():
 
     import torch
 
-    from oracle import moe as OM
     from pith_train_amd import _lib
     from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
     from pith_train_amd.modules.experts import forward_stage3
@@ -342,7 +358,7 @@ def main():
         expand_idx = expand_cpu.cuda()
     else:
         tokens = x.cuda().unsqueeze(1).expand(-1, k, -1).reshape(-1, H).contiguous()
-    flops = OM.gemm_flops(rows, H, I) + extra_flops(extras, T, H)
+    flops = gemm_flops(rows, H, I) + extra_flops(extras, T, H)
     dense = []  # (module, input [T, in], upstream grad [T, out])
     if extras.get("shared_mlp") or extras.get("dense_linears"):
         from pith_train_amd.modules import training
