@@ -132,7 +132,8 @@ def build_module(kind, H, I, E, w):
 class GemmTimer:
     """HIP events (on the stream the kernels are launched on) around every GEMM entry point."""
 
-    NAMES = ("pt_gemm_m_grouped_nt", "pt_gemm_m_grouped_nt_scatter", "pt_gemm_k_grouped_wgrad", "pt_gemm_nt_dense")
+    NAMES = ("pt_gemm_m_grouped_nt", "pt_gemm_m_grouped_nt_scatter", "pt_gemm_k_grouped_wgrad", "pt_gemm_k_grouped_wgrad_ld",
+             "pt_gemm_nt_dense")
 
     def __init__(self):
         self.records = []
@@ -154,7 +155,8 @@ class GemmTimer:
                 orig(name, *args)
                 b.record()
                 # rows x columns x reduction as the entry point takes them (the three int64 sizes)
-                sizes = {"pt_gemm_nt_dense": args[6:9], "pt_gemm_k_grouped_wgrad": args[9:12]}.get(name, args[8:11])
+                sizes = {"pt_gemm_nt_dense": args[6:9], "pt_gemm_k_grouped_wgrad": args[9:12],
+                         "pt_gemm_k_grouped_wgrad_ld": args[11:14]}.get(name, args[8:11])
                 timer.records.append((name, a, b, "x".join(str(int(v)) for v in sizes)))
             else:
                 orig(name, *args)
@@ -192,7 +194,7 @@ class GemmTimer:
                 flop = 2.0 * real * nn * k
                 # (m may be the buffers' capacity rather than the padded row count, which then only
                 # the device knows: the floor counts the rows that carry tokens)
-                if name == "pt_gemm_k_grouped_wgrad":  # dW[g] = dY_g^T X_g: both twins read, [G,N,K] written
+                if name.startswith("pt_gemm_k_grouped_wgrad"):  # dW[g] = dY_g^T X_g: both twins read, [G,N,K] written
                     byts = real * (nn + k) * (1 + 4 / 128) + 2.0 * groups * nn * k
                 else:
                     byts = real * k * (1 + 4 / 128) + groups * nn * k * (1 + 4 / 16384) + 2.0 * real * nn

@@ -102,6 +102,17 @@ int pt_quant_blockwise_transpose_batched(const void* x, int dtype, int64_t G, in
                                          int64_t stride_g, int64_t stride_row, void* fp8,
                                          float* scale, void* fp8_t, float* scale_t,
                                          pt_stream_t stream);
+/* The same into slices of larger outputs: group strides for fp8 / scale, and for the transposed
+ * twin its row pitch t_ld (>= N), group stride, and the row length scale_t_ld of its scale grid.
+ * Separate gate and up weights are quantised into one fused [G, 2I, K] operand this way (the up
+ * half starts I rows, i.e. I*K bytes / I columns of the twin, further in). */
+int pt_quant_blockwise_transpose_batched_into(const void* x, int dtype, int64_t G, int64_t N,
+                                              int64_t K, int64_t stride_g, int64_t stride_row,
+                                              void* fp8, int64_t fp8_stride_g, float* scale,
+                                              int64_t scale_stride_g, void* fp8_t, int64_t t_ld,
+                                              int64_t t_stride_g, float* scale_t,
+                                              int64_t scale_t_ld, int64_t scale_t_stride_g,
+                                              pt_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * FP8 GEMMs (fp32 accumulate on the MFMA units, scales applied in hardware as E8M0).
@@ -146,6 +157,14 @@ int pt_gemm_k_grouped_wgrad(const void* dy_t_fp8, const float* dy_scale, const v
                             const float* x_scale, void* out, int out_dtype, int accumulate,
                             const int32_t* offs, int32_t num_groups, int64_t M, int64_t N,
                             int64_t K, pt_stream_t stream);
+/* The same with the row length of the two scale arrays given: dy_scale[M/128, ld_dy_scale] and
+ * x_scale[M/128, ld_x_scale] may be column slices of wider arrays (the gate and up halves of a
+ * fused projection's colwise twin get their own weight-gradient tensors this way). */
+int pt_gemm_k_grouped_wgrad_ld(const void* dy_t_fp8, const float* dy_scale, int64_t ld_dy_scale,
+                               const void* x_t_fp8, const float* x_scale, int64_t ld_x_scale,
+                               void* out, int out_dtype, int accumulate, const int32_t* offs,
+                               int32_t num_groups, int64_t M, int64_t N, int64_t K,
+                               pt_stream_t stream);
 
 /* Which GEMM kernel the three entry points above launch: "auto" (or NULL: per call from the
  * shape; the default unless the environment variable PT_GEMM_IMPL names one of the others),

@@ -33,10 +33,13 @@ SIGNATURES = {
     "pt_quant_rowwise_transpose": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, P]),
     "pt_quant_rowwise_blockwise_transpose": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, P]),
     "pt_quant_blockwise_transpose_batched": (c_int, [P, c_int, I64, I64, I64, I64, I64, P, P, P, P, P]),
+    "pt_quant_blockwise_transpose_batched_into": (c_int, [P, c_int, I64, I64, I64, I64, I64, P, I64, P, I64, P, I64, I64, P, I64,
+                                                          I64, P]),
     "pt_gemm_nt_dense": (c_int, [P, P, P, P, P, c_int, I64, I64, I64, P]),
     "pt_gemm_m_grouped_nt": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P]),
     "pt_gemm_m_grouped_nt_scatter": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, I64, P]),
     "pt_gemm_k_grouped_wgrad": (c_int, [P, P, P, P, P, c_int, c_int, P, I32, I64, I64, I64, P]),
+    "pt_gemm_k_grouped_wgrad_ld": (c_int, [P, P, I64, P, P, I64, P, c_int, c_int, P, I32, I64, I64, I64, P]),
     "pt_gemm_select_kernel": (c_int, [ctypes.c_char_p]),
     "pt_moe_combine_fwd": (c_int, [P, I64, P, P, I64, P, I64, I64, I32, I64, c_int, P]),
     "pt_moe_combine_bwd": (c_int, [P, I64, P, I64, P, P, I64, P, I64, I32, I64, c_int, P]),

@@ -386,9 +386,9 @@ extern "C" int pt_gemm_m_grouped_nt_scatter(const void* a_fp8, const float* a_sc
   return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, out_row_index, out_rows, stream);
 }
 
-extern "C" int pt_gemm_k_grouped_wgrad(const void* dy_t_fp8, const float* dy_scale, const void* x_t_fp8, const float* x_scale,
-                                       void* out, int out_dtype, int accumulate, const int32_t* offs, int32_t G, int64_t M,
-                                       int64_t N, int64_t K, pt_stream_t stream) {
+static int gemm_k_grouped_wgrad_impl(const void* dy_t_fp8, const float* dy_scale, int64_t ld_dy_scale, const void* x_t_fp8,
+                                     const float* x_scale, int64_t ld_x_scale, void* out, int out_dtype, int accumulate,
+                                     const int32_t* offs, int32_t G, int64_t M, int64_t N, int64_t K, pt_stream_t stream) {
   PT_REQUIRE(M >= 0 && N >= 0 && K >= 0 && G > 0, "gemm_k_grouped_wgrad: bad sizes");
   if (N == 0 || K == 0) return PT_OK;
   PT_REQUIRE(M % 128 == 0, "gemm_k_grouped_wgrad: M=%lld must be a multiple of 128", (long long)M);
@@ -396,15 +396,30 @@ extern "C" int pt_gemm_k_grouped_wgrad(const void* dy_t_fp8, const float* dy_sca
   PT_REQUIRE(M == 0 || (dy_t_fp8 && dy_scale && x_t_fp8 && x_scale && al16(dy_t_fp8) && al16(x_t_fp8)),
              "gemm_k_grouped_wgrad: null or misaligned pointer");
   PT_REQUIRE(out_dtype == PT_BF16 || out_dtype == PT_F32, "gemm_k_grouped_wgrad: out_dtype must be bf16 or fp32");
+  PT_REQUIRE(ld_dy_scale >= N && ld_x_scale >= K, "gemm_k_grouped_wgrad: scale row length smaller than the row count");
   GemmArgs g = {};
   g.a = (const uint8_t*)dy_t_fp8; g.lda = M; g.b = (const uint8_t*)x_t_fp8; g.ldb = M;
-  g.sa = dy_scale; g.sa_rs = 1; g.sa_ks = N; g.sa_shift = 0;
-  g.sb = x_scale; g.sb_rs = 1; g.sb_ks = K; g.sb_shift = 0;
+  g.sa = dy_scale; g.sa_rs = 1; g.sa_ks = ld_dy_scale; g.sa_shift = 0;
+  g.sb = x_scale; g.sb_rs = 1; g.sb_ks = ld_x_scale; g.sb_shift = 0;
   g.out = out; g.ldo = K; g.out_dtype = out_dtype; g.accumulate = accumulate;
   g.rows_a = N; g.rows_b = K; g.red = M; g.mode = GEMM_K_GROUPED; g.offs = offs; g.G = G;
   g.out_stride_g = N * K;
-  g.a_bytes = N * M; g.b_bytes = K * M; g.sa_bytes = (M / 128) * N * 4; g.sb_bytes = (M / 128) * K * 4;
+  g.a_bytes = N * M; g.b_bytes = K * M;
+  g.sa_bytes = ((M / 128 - 1) * ld_dy_scale + N) * 4; g.sb_bytes = ((M / 128 - 1) * ld_x_scale + K) * 4;
   g.tiles_a = (int)cdiv(N, 128); g.tiles_b = (int)cdiv(K, 128);
   g.total_tiles = (int64_t)g.tiles_a * g.tiles_b * G;
   return dispatch_gemm(g, (hipStream_t)stream);
+}
+
+extern "C" int pt_gemm_k_grouped_wgrad(const void* dy_t_fp8, const float* dy_scale, const void* x_t_fp8, const float* x_scale,
+                                       void* out, int out_dtype, int accumulate, const int32_t* offs, int32_t G, int64_t M,
+                                       int64_t N, int64_t K, pt_stream_t stream) {
+  return gemm_k_grouped_wgrad_impl(dy_t_fp8, dy_scale, N, x_t_fp8, x_scale, K, out, out_dtype, accumulate, offs, G, M, N, K, stream);
+}
+
+extern "C" int pt_gemm_k_grouped_wgrad_ld(const void* dy_t_fp8, const float* dy_scale, int64_t ld_dy_scale, const void* x_t_fp8,
+                                          const float* x_scale, int64_t ld_x_scale, void* out, int out_dtype, int accumulate,
+                                          const int32_t* offs, int32_t G, int64_t M, int64_t N, int64_t K, pt_stream_t stream) {
+  return gemm_k_grouped_wgrad_impl(dy_t_fp8, dy_scale, ld_dy_scale, x_t_fp8, x_scale, ld_x_scale, out, out_dtype, accumulate,
+                                   offs, G, M, N, K, stream);
 }

@@ -34,6 +34,8 @@ struct QuantArgs {
   const void* x2; int64_t ldx2;  // fused SwiGLU backward: the saved gate_up [M, 2*half]
   int64_t half;                  // fused SwiGLU: width of one half of gate_up
   const int32_t* row_limit;      // optional device scalar: row tiles at or past *row_limit are skipped (nothing written)
+  int64_t ld_t;                  // row pitch of the transposed twin (bytes = elements); M unless it is a column slice
+  int64_t bs_ld;                 // row length of the twin's block-scale grid; tiles_m unless it is a column slice
 };
 
 template <typename T> struct Loader;
@@ -404,7 +406,7 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
   } else {
 #pragma unroll
     for (int j = 0; j < 8; ++j) { crcp[j] = blk_rcp; cs[j] = blk_scale; }
-    if (t == 0) p.b_scale[g * p.b_scale_stride_g + (int64_t)tc * p.tiles_m + tr] = blk_scale;
+    if (t == 0) p.b_scale[g * p.b_scale_stride_g + (int64_t)tc * p.bs_ld + tr] = blk_scale;
   }
 
   if (BL == BL_ROWMAJOR) {
@@ -467,8 +469,8 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
     uint8_t* base;
     int64_t ld;
     if (BL == BL_TRANSPOSED) {
-      base = p.b_out + g * p.b_stride_g + (int64_t)tc * 128 * p.M + (int64_t)tr * 128;
-      ld = p.M;
+      base = p.b_out + g * p.b_stride_g + (int64_t)tc * 128 * p.ld_t + (int64_t)tr * 128;
+      ld = p.ld_t;
     } else {
       const int64_t row_start = (int64_t)tr * 128;
       int grp = 0;
@@ -554,7 +556,7 @@ static void fill_common(QuantArgs& a, const void* x, int dtype, int64_t M, int64
   a.a_stride_g = 0; a.a_scale_stride_g = 0; a.b_stride_g = 0; a.b_scale_stride_g = 0;
   a.tiles_m = (int32_t)cdiv(M, 128); a.tiles_n = (int32_t)cdiv(N, 128);
   a.offs = nullptr; a.num_groups = 0; a.row_index = nullptr; a.x2 = nullptr; a.ldx2 = 0; a.half = 0;
-  a.row_limit = nullptr;
+  a.row_limit = nullptr; a.ld_t = M; a.bs_ld = a.tiles_m;
   const int eb = dtype == PT_F32 ? 4 : 2;
   a.vec_in = (N % 8 == 0) && ((ldx * eb) % 16 == 0) && (((uintptr_t)x) % 16 == 0);
   a.vec_out = (N % 8 == 0);
@@ -635,24 +637,47 @@ extern "C" int pt_quant_rowwise_blockwise_transpose(const void* x, int dtype, in
   return launch_quant<A_ROW, B_BLOCK, BL_TRANSPOSED, BS_MB_N>(a, dtype, 1, (hipStream_t)stream);
 }
 
-extern "C" int pt_quant_blockwise_transpose_batched(const void* x, int dtype, int64_t G, int64_t N,
-                                                    int64_t K, int64_t stride_g, int64_t stride_row,
-                                                    void* fp8, float* scale, void* fp8_t,
-                                                    float* scale_t, pt_stream_t stream) {
+static int quant_blockwise_transpose_batched_impl(const void* x, int dtype, int64_t G, int64_t N, int64_t K, int64_t stride_g,
+                                                  int64_t stride_row, void* fp8, int64_t fp8_stride_g, float* scale,
+                                                  int64_t scale_stride_g, void* fp8_t, int64_t t_ld, int64_t t_stride_g,
+                                                  float* scale_t, int64_t scale_t_ld, int64_t scale_t_stride_g,
+                                                  pt_stream_t stream) {
   PT_REQUIRE(G >= 0 && N >= 0 && K >= 0 && stride_row >= K, "quant_blockwise_transpose_batched: bad shape");
   if (G == 0 || N == 0 || K == 0) return PT_OK;
   PT_REQUIRE(x && fp8 && scale && fp8_t && scale_t, "quant_blockwise_transpose_batched: null pointer");
   QuantArgs a;
   fill_common(a, x, dtype, N, K, stride_row);
+  PT_REQUIRE(fp8_stride_g >= N * K && t_ld >= N && t_stride_g >= K * t_ld - (t_ld - N) && scale_t_ld >= a.tiles_m,
+             "quant_blockwise_transpose_batched: output strides smaller than the tensors");
   const int eb = dtype == PT_F32 ? 4 : 2;
   a.vec_in = a.vec_in && ((stride_g * eb) % 16 == 0);
   a.x_stride_g = stride_g;
-  a.a_out = (uint8_t*)fp8; a.a_stride_g = N * K; a.a_scale = scale; a.a_scale_stride_g = (int64_t)a.tiles_m * a.tiles_n;
-  a.b_out = (uint8_t*)fp8_t; a.b_stride_g = N * K; a.b_scale = scale_t; a.b_scale_stride_g = (int64_t)a.tiles_m * a.tiles_n;
-  // transposed stores of group g start at g*N*K: 16-byte alignment needs (N*K) % 16 == 0 too
-  a.vec_out_t = a.vec_out_t && ((N * K) % 16 == 0);
-  a.vec_out = a.vec_out && ((N * K) % 8 == 0);
+  a.a_out = (uint8_t*)fp8; a.a_stride_g = fp8_stride_g; a.a_scale = scale; a.a_scale_stride_g = scale_stride_g;
+  a.b_out = (uint8_t*)fp8_t; a.b_stride_g = t_stride_g; a.b_scale = scale_t; a.b_scale_stride_g = scale_t_stride_g;
+  a.ld_t = t_ld; a.bs_ld = scale_t_ld;
+  // 16-byte transposed stores need every row start aligned: the pitch, the group stride and the base
+  a.vec_out_t = a.vec_out_t && (t_ld % 16 == 0) && (t_stride_g % 16 == 0) && (((uintptr_t)fp8_t) % 16 == 0);
+  a.vec_out = a.vec_out && (fp8_stride_g % 8 == 0) && (((uintptr_t)fp8) % 8 == 0);
   return launch_quant<A_BLOCK, B_BLOCK, BL_TRANSPOSED, BS_MB_N>(a, dtype, G, (hipStream_t)stream);
+}
+
+extern "C" int pt_quant_blockwise_transpose_batched(const void* x, int dtype, int64_t G, int64_t N,
+                                                    int64_t K, int64_t stride_g, int64_t stride_row,
+                                                    void* fp8, float* scale, void* fp8_t,
+                                                    float* scale_t, pt_stream_t stream) {
+  const int64_t nb = cdiv(N, 128), kb = cdiv(K, 128);
+  return quant_blockwise_transpose_batched_impl(x, dtype, G, N, K, stride_g, stride_row, fp8, N * K, scale, nb * kb, fp8_t, N,
+                                                N * K, scale_t, nb, nb * kb, stream);
+}
+
+extern "C" int pt_quant_blockwise_transpose_batched_into(const void* x, int dtype, int64_t G, int64_t N, int64_t K,
+                                                         int64_t stride_g, int64_t stride_row, void* fp8,
+                                                         int64_t fp8_stride_g, float* scale, int64_t scale_stride_g,
+                                                         void* fp8_t, int64_t t_ld, int64_t t_stride_g, float* scale_t,
+                                                         int64_t scale_t_ld, int64_t scale_t_stride_g, pt_stream_t stream) {
+  return quant_blockwise_transpose_batched_impl(x, dtype, G, N, K, stride_g, stride_row, fp8, fp8_stride_g, scale,
+                                                scale_stride_g, fp8_t, t_ld, t_stride_g, scale_t, scale_t_ld,
+                                                scale_t_stride_g, stream);
 }
 
 // ---- SwiGLU fused into the activation quantisation --------------------------------------------

@@ -22,7 +22,7 @@ import torch.nn as nn
 from ..dualpipe_utils import FP8WeightCacheControl
 from ..operators import fused_experts
 from ..operators.clamped_swiglu import clamped_swiglu
-from ..operators.deepgemm_quantize import fp8cast_blockwise_transpose_batched
+from ..operators.deepgemm_quantize import fp8cast_blockwise_transpose_batched, fp8cast_blockwise_transpose_batched_cat
 from ..operators.grouped_linear import FP8GroupedLinear, FP8GroupedLinearFunc, GroupedLinearFunc
 from ..operators.indexed_bias_add import indexed_bias_add
 from ..operators.silu_mul import silu_mul, silu_mul_halves
@@ -43,10 +43,33 @@ class Qwen3MoeExperts(nn.Module):
         self.up_proj = training.GroupedLinear(num_experts, hidden_size, moe_intermediate_size)
         self.down_proj = training.GroupedLinear(num_experts, moe_intermediate_size, hidden_size)
 
-    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None):
+    def _fused_gate_up_quant(self):
+        """gate and up weights quantised into one fused ``[G, 2I, H]`` operand; cached like the
+        layers' own quantised weights (one quantisation per ``FP8WeightCacheControl`` version)."""
+        parts = [self.gate_proj.weight, self.up_proj.weight]
+        if torch.compiler.is_compiling():
+            return fp8cast_blockwise_transpose_batched_cat(parts)
+        ver = FP8WeightCacheControl.version
+        if getattr(self, "_gu_cache", None) is None or self._gu_version != ver:
+            self._gu_cache = fp8cast_blockwise_transpose_batched_cat(parts)
+            self._gu_version = ver
+        return self._gu_cache
+
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None, fuse_activation: bool = True):
         """``row_map`` (extension, FP8 layers only): the scatter's int32 source-row map.  ``x`` is
         then the un-permuted ``[m, H]`` token tensor and the result comes back un-permuted; the
-        permutation happens inside the first quantisation and the last GEMM's store."""
+        permutation happens inside the first quantisation and the last GEMM's store.  With
+        ``fuse_activation`` (FP8 layers, intermediate size a multiple of 128) the block runs as one
+        autograd node on a fused gate_up operand: the tokens are quantised once instead of once
+        per projection, one GEMM serves both, and the SwiGLU and its gradient are computed inside
+        the kernels that quantise them (same bits as the three-operator composition)."""
+        if (fuse_activation and training.fp8 and x.shape[0] > 0 and isinstance(self.gate_proj, FP8GroupedLinear)
+                and isinstance(self.up_proj, FP8GroupedLinear) and isinstance(self.down_proj, FP8GroupedLinear)
+                and fused_experts.supported_split(x, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight)):
+            return fused_experts.FP8SwiGLUSplitExpertsFunc.apply(
+                x, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight, grouped_mm_offs,
+                self._fused_gate_up_quant(), self.down_proj._get_quantized_weight(), row_map,
+            )  # fmt: skip
         gi = precompute_group_indices(grouped_mm_offs, x.shape[0])
         kwargs = dict(grouped_mm_offs=grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, group_indices=gi)
         if row_map is not None:
@@ -174,8 +197,12 @@ def forward_stage3(experts: nn.Module, gathered_tokens, expert_idxs, experts_per
             and isinstance(experts, (Qwen3MoeExperts, Qwen35MoeExperts))
             and isinstance(experts.down_proj, FP8GroupedLinear)
             and experts.down_proj.out_features % 8 == 0 and experts.down_proj.in_features % 8 == 0):
-        fused_node = isinstance(experts, Qwen35MoeExperts) and fused_experts.supported(
-            gathered_tokens, experts.gate_up_proj.weight, experts.down_proj.weight)
+        if isinstance(experts, Qwen35MoeExperts):
+            fused_node = fused_experts.supported(gathered_tokens, experts.gate_up_proj.weight, experts.down_proj.weight)
+        else:
+            fused_node = (isinstance(experts.gate_proj, FP8GroupedLinear) and isinstance(experts.up_proj, FP8GroupedLinear)
+                          and fused_experts.supported_split(gathered_tokens, experts.gate_proj.weight,
+                                                            experts.up_proj.weight, experts.down_proj.weight))
         _, grouped_mm_offs, ks, ks_tensor, src_of = group_rows_with_sizes(
             expert_idxs, experts_per_rank, device=gathered_tokens.device, host_sizes=host_sizes or not fused_node)
         return experts(gathered_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, row_map=src_of)

@@ -167,6 +167,37 @@ def _blockwise_batched(x3: torch.Tensor):
     return out, scale, out_t, scale_t
 
 
+def fp8cast_blockwise_transpose_batched_cat(parts):
+    """:func:`fp8cast_blockwise_transpose_batched` of ``torch.cat(parts, dim=1)`` without the
+    concatenation: each ``[G, N_i, K]`` part is quantised straight into its rows of the fused
+    outputs (and its columns of the transposed twin).  ``N_i % 128 == 0`` so that the 128x128
+    blocks of the fused tensor are blocks of the parts; separate gate and up weights become one
+    fused projection operand this way."""
+    G, _, K = parts[0].shape
+    dev = parts[0].device
+    assert all(p_.ndim == 3 and p_.shape[0] == G and p_.shape[2] == K and p_.shape[1] % 128 == 0 for p_ in parts)
+    N = sum(p_.shape[1] for p_ in parts)
+    nb, kb = N // 128, _cdiv(K, 128)
+    out = torch.empty((G, N, K), dtype=FP8, device=dev)
+    scale = torch.empty((G, nb, kb), dtype=torch.float32, device=dev)
+    out_t = torch.empty((G, K, N), dtype=FP8, device=dev)
+    scale_t = torch.empty((G, kb, nb), dtype=torch.float32, device=dev)
+    row = 0
+    for part in parts:
+        x3 = _prep2d(part.detach())
+        n = x3.shape[1]
+        if G and n and K:
+            _lib.call(
+                "pt_quant_blockwise_transpose_batched_into", x3.data_ptr(), _lib.dtype_code(x3.dtype), G, n, K,
+                x3.stride(0) if G > 1 else n * K, x3.stride(1) if n > 1 else K,
+                out.data_ptr() + row * K, N * K, scale.data_ptr() + 4 * (row // 128) * kb, nb * kb,
+                out_t.data_ptr() + row, N, K * N, scale_t.data_ptr() + 4 * (row // 128), nb, kb * nb,
+                _lib.stream_ptr(dev),
+            )  # fmt: skip
+        row += n
+    return out, scale, out_t, scale_t
+
+
 def fp8cast_blockwise_transpose(x: torch.Tensor):
     """(fp8[M,K], scale[ceil(M/128),ceil(K/128)], fp8_t[K,M], scale_t[ceil(K/128),ceil(M/128)])."""
     assert x.ndim == 2, f"Expected 2D tensor, got {x.ndim}D"

@@ -71,6 +71,65 @@ def supported(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) ->
             and w_down.shape[1] % 8 == 0 and w_down.shape[2] == half)
 
 
+def _forward(ctx, x, gate_up_weights, w_down, grouped_mm_offs, q_gate_up, q_down, row_map):
+    """Shared forward of the two autograd nodes below.  ``gate_up_weights``: the parameters whose
+    gradients the gate_up weight gradient is written to, one fused ``[G, 2I, K]`` tensor or the
+    pair ``(gate [G, I, K], up [G, I, K])``."""
+    _lib.require_cuda(x)
+    gu_fp8, gu_scale, gu_t_fp8, gu_t_scale = q_gate_up
+    dn_fp8, dn_scale, dn_t_fp8, dn_t_scale = q_down
+    two_i = gu_fp8.shape[1]
+    H = w_down.shape[1]
+    if row_map is not None:
+        M = row_map.shape[0]
+        x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, row_map, grouped_mm_offs)
+    else:
+        M = x.shape[0]
+        x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t(x)
+    gate_up = torch.empty((M, two_i), device=x.device, dtype=x.dtype)
+    m_grouped_fp8_gemm_nt((x_fp8, x_s), (gu_fp8, gu_scale), gate_up, grouped_mm_offs)
+    del x_fp8, x_s
+    h_fp8, h_s, h_ch_t, h_ch_s = silu_mul_quant(gate_up, grouped_mm_offs if row_map is not None else None)
+    out = torch.empty((x.shape[0], H), device=x.device, dtype=x.dtype)
+    m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, row_map)
+    ctx.save_for_backward(gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, grouped_mm_offs, x_ch_t, x_ch_s,
+                          gate_up, h_ch_t, h_ch_s, row_map)
+    ctx.gate_up_weights, ctx.w_down = gate_up_weights, w_down
+    ctx.rows = (M, x.shape[0])
+    return out
+
+
+def _backward(ctx, grad_out):
+    """Shared backward: returns the gradient of ``x``; the weight gradients go to ``.grad`` (or to
+    the ``WeightGradStore`` queue) through :func:`schedule_wgrad`."""
+    (gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, offs, x_ch_t, x_ch_s, gate_up, h_ch_t, h_ch_s,
+     row_map) = ctx.saved_tensors  # fmt: skip
+    M, rows_x = ctx.rows
+    half = gate_up.shape[1] // 2
+    K = gu_t_fp8.shape[1]
+    grad_out = grad_out.contiguous()
+    if row_map is not None:
+        dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t_rows(grad_out, row_map, offs)
+    else:
+        dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t(grad_out)
+    grad_h = torch.empty((M, half), device=grad_out.device, dtype=grad_out.dtype)
+    m_grouped_fp8_gemm_nt((dy_fp8, dy_s), (dn_t_fp8, dn_t_scale), grad_h, offs)
+    schedule_wgrad(ctx.w_down, (dy_ch_t, dy_ch_s), (h_ch_t, h_ch_s), offs)
+    del dy_fp8, dy_s
+    dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s = silu_mul_bwd_quant(grad_h, gate_up, offs if row_map is not None else None)
+    grad_x = torch.empty((rows_x, K), device=grad_out.device, dtype=grad_out.dtype)
+    m_grouped_fp8_gemm_nt((dgu_fp8, dgu_s), (gu_t_fp8, gu_t_scale), grad_x, offs, row_map)
+    if isinstance(ctx.gate_up_weights, tuple):
+        # separate gate and up parameters: each gets the weight-gradient GEMM of its half of the
+        # colwise twin (rows of the transposed bytes, columns of the scale array)
+        w_gate, w_up = ctx.gate_up_weights
+        schedule_wgrad(w_gate, (dgu_ch_t[:half], dgu_ch_s[:, :half]), (x_ch_t, x_ch_s), offs)
+        schedule_wgrad(w_up, (dgu_ch_t[half:], dgu_ch_s[:, half:]), (x_ch_t, x_ch_s), offs)
+    else:
+        schedule_wgrad(ctx.gate_up_weights, (dgu_ch_t, dgu_ch_s), (x_ch_t, x_ch_s), offs)
+    return grad_x
+
+
 class FP8SwiGLUExpertsFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, w_gate_up, w_down, grouped_mm_offs, ks, ks_tensor, q_gate_up, q_down, row_map=None):
@@ -78,48 +137,31 @@ class FP8SwiGLUExpertsFunc(torch.autograd.Function):
         ``[m, K]`` tokens; the result has the same row layout as ``x``.  ``row_map`` may be longer
         than the grouped rows (its tail negative): every kernel takes the real row count from
         ``grouped_mm_offs`` on the device, so no host-side size is needed (``ks`` may be None)."""
-        _lib.require_cuda(x)
-        gu_fp8, gu_scale, gu_t_fp8, gu_t_scale = q_gate_up
-        dn_fp8, dn_scale, dn_t_fp8, dn_t_scale = q_down
-        num_groups, two_i, K = w_gate_up.shape
-        H = w_down.shape[1]
-        if row_map is not None:
-            M = row_map.shape[0]
-            x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, row_map, grouped_mm_offs)
-        else:
-            M = x.shape[0]
-            x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t(x)
-        gate_up = torch.empty((M, two_i), device=x.device, dtype=x.dtype)
-        m_grouped_fp8_gemm_nt((x_fp8, x_s), (gu_fp8, gu_scale), gate_up, grouped_mm_offs)
-        del x_fp8, x_s
-        h_fp8, h_s, h_ch_t, h_ch_s = silu_mul_quant(gate_up, grouped_mm_offs if row_map is not None else None)
-        out = torch.empty((x.shape[0], H), device=x.device, dtype=x.dtype)
-        m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, row_map)
-        ctx.save_for_backward(gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, grouped_mm_offs, x_ch_t, x_ch_s,
-                              gate_up, h_ch_t, h_ch_s, row_map)
-        ctx.w_gate_up, ctx.w_down = w_gate_up, w_down
-        ctx.rows = (M, x.shape[0])
-        return out
+        return _forward(ctx, x, w_gate_up, w_down, grouped_mm_offs, q_gate_up, q_down, row_map)
 
     @staticmethod
     def backward(ctx, grad_out):
-        (gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, offs, x_ch_t, x_ch_s, gate_up, h_ch_t, h_ch_s,
-         row_map) = ctx.saved_tensors  # fmt: skip
-        w_gate_up, w_down = ctx.w_gate_up, ctx.w_down
-        M, rows_x = ctx.rows
-        half = gate_up.shape[1] // 2
-        K = w_gate_up.shape[2]
-        grad_out = grad_out.contiguous()
-        if row_map is not None:
-            dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t_rows(grad_out, row_map, offs)
-        else:
-            dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t(grad_out)
-        grad_h = torch.empty((M, half), device=grad_out.device, dtype=grad_out.dtype)
-        m_grouped_fp8_gemm_nt((dy_fp8, dy_s), (dn_t_fp8, dn_t_scale), grad_h, offs)
-        schedule_wgrad(w_down, (dy_ch_t, dy_ch_s), (h_ch_t, h_ch_s), offs)
-        del dy_fp8, dy_s
-        dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s = silu_mul_bwd_quant(grad_h, gate_up, offs if row_map is not None else None)
-        grad_x = torch.empty((rows_x, K), device=grad_out.device, dtype=grad_out.dtype)
-        m_grouped_fp8_gemm_nt((dgu_fp8, dgu_s), (gu_t_fp8, gu_t_scale), grad_x, offs, row_map)
-        schedule_wgrad(w_gate_up, (dgu_ch_t, dgu_ch_s), (x_ch_t, x_ch_s), offs)
-        return grad_x, None, None, None, None, None, None, None, None
+        return _backward(ctx, grad_out), None, None, None, None, None, None, None, None
+
+
+class FP8SwiGLUSplitExpertsFunc(torch.autograd.Function):
+    """The same node for experts that keep gate and up as separate parameters
+    (``Qwen3MoeExperts`` / ``DeepSeekV2Experts``, models/qwen3_moe.py:45-65): ``q_gate_up`` is the
+    two weights quantised into one fused operand (:func:`fp8cast_blockwise_transpose_batched_cat`),
+    so the tokens are quantised once and one GEMM each way serves both projections; the weight
+    gradients are written to the two parameters separately."""
+
+    @staticmethod
+    def forward(ctx, x, w_gate, w_up, w_down, grouped_mm_offs, q_gate_up, q_down, row_map=None):
+        return _forward(ctx, x, (w_gate, w_up), w_down, grouped_mm_offs, q_gate_up, q_down, row_map)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        return _backward(ctx, grad_out), None, None, None, None, None, None, None
+
+
+def supported_split(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> bool:
+    """As :func:`supported`, and the halves must be whole 128-row blocks of the fused operand."""
+    half = w_gate.shape[1]
+    return (x.dtype == torch.bfloat16 and w_gate.shape == w_up.shape and half % 128 == 0
+            and w_down.shape[1] % 8 == 0 and w_down.shape[2] == half)

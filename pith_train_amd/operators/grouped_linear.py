@@ -130,16 +130,28 @@ def m_grouped_fp8_gemm_nt(a, b, out: torch.Tensor, grouped_mm_offs: torch.Tensor
 
 
 def k_grouped_fp8_wgrad(dy_t, x_t, out: torch.Tensor, grouped_mm_offs, accumulate: bool):
-    """out[g] (+)= dY_g^T X_g with dy_t=(fp8[N,M], scale[M/128,N]), x_t=(fp8[K,M], scale[M/128,K])."""
+    """out[g] (+)= dY_g^T X_g with dy_t=(fp8[N,M], scale[M/128,N]), x_t=(fp8[K,M], scale[M/128,K]).
+    The fp8 operands are contiguous; the scale arrays may be column slices of wider arrays (their
+    row stride is passed on)."""
     (dy_fp8, dy_s), (x_fp8, x_s) = dy_t, x_t
     N, M = dy_fp8.shape
     K = x_fp8.shape[0]
     G = out.shape[0]
-    _lib.call(
-        "pt_gemm_k_grouped_wgrad", dy_fp8.data_ptr(), dy_s.data_ptr(), x_fp8.data_ptr(),
-        x_s.data_ptr(), out.data_ptr(), _lib.dtype_code(out.dtype), int(accumulate),
-        grouped_mm_offs.data_ptr(), G, M, N, K, _lib.stream_ptr(out.device),
-    )  # fmt: skip
+    assert dy_fp8.is_contiguous() and x_fp8.is_contiguous() and dy_s.stride(-1) == 1 and x_s.stride(-1) == 1
+    ld_dy = dy_s.stride(0) if dy_s.shape[0] > 1 else N
+    ld_x = x_s.stride(0) if x_s.shape[0] > 1 else K
+    if ld_dy == N and ld_x == K:
+        _lib.call(
+            "pt_gemm_k_grouped_wgrad", dy_fp8.data_ptr(), dy_s.data_ptr(), x_fp8.data_ptr(),
+            x_s.data_ptr(), out.data_ptr(), _lib.dtype_code(out.dtype), int(accumulate),
+            grouped_mm_offs.data_ptr(), G, M, N, K, _lib.stream_ptr(out.device),
+        )  # fmt: skip
+    else:
+        _lib.call(
+            "pt_gemm_k_grouped_wgrad_ld", dy_fp8.data_ptr(), dy_s.data_ptr(), ld_dy, x_fp8.data_ptr(),
+            x_s.data_ptr(), ld_x, out.data_ptr(), _lib.dtype_code(out.dtype), int(accumulate),
+            grouped_mm_offs.data_ptr(), G, M, N, K, _lib.stream_ptr(out.device),
+        )  # fmt: skip
     return out
 
 

@@ -116,20 +116,24 @@ def test_stage3_permute_folded_into_quant_and_gemm_is_bit_identical(kind, E, H, 
     for fuse, fuse_act, host_sizes in ((True, True, False), (True, True, True), (False, False, True), (False, True, True),
                                        (True, False, True)):
         mod, params = _build(kind, E, H, I, w)
-        if kind == "fused":  # the one-node SwiGLU block exists for the fused gate_up layout
-            mod.forward = functools.partial(mod.forward, fuse_activation=fuse_act)
-        elif fuse_act != fuse:
-            continue
+        mod.forward = functools.partial(mod.forward, fuse_activation=fuse_act)
         FP8WeightCacheControl.step()
         tok = tokens.clone().requires_grad_(True)
         out = forward_stage3(mod, tok, ids.reshape(-1).cuda(), E, fuse_permute=fuse, host_sizes=host_sizes)
         out.backward(dy)
-        res.append((out.detach(), tok.grad, {n: p.grad for n, p in params.items()}))
+        res.append((fuse_act, out.detach(), tok.grad, {n: p.grad for n, p in params.items()}))
     for other in res[1:]:
-        assert torch.equal(res[0][0], other[0]), "forward output differs"
-        assert torch.equal(res[0][1], other[1]), "token gradient differs"
-        for n in res[0][2]:
-            assert torch.equal(res[0][2][n], other[2][n]), f"{n} gradient differs"
+        assert torch.equal(res[0][1], other[1]), "forward output differs"
+        for n in res[0][3]:
+            assert torch.equal(res[0][3][n], other[3][n]), f"{n} gradient differs"
+        if kind == "fused" or other[0] == res[0][0]:
+            assert torch.equal(res[0][2], other[2]), "token gradient differs"
+        else:
+            # Separate gate and up parameters: the three-operator composition adds two bf16 token
+            # gradients (one per projection, as the reference does), the one-node path accumulates
+            # both halves in one fp32 GEMM sum and rounds once.
+            a, b = res[0][2].float(), other[2].float()
+            assert ((a - b).abs() <= 2.0**-6 * b.abs().amax(dim=1, keepdim=True)).all(), "token gradient differs"
 
 
 def test_stage3_with_dedup_expand_fused_and_unfused():
