@@ -191,3 +191,25 @@ def test_k_grouped_wgrad(sizes, N, K, accumulate):
         out32 = old32.clone().cuda()
         k_grouped_fp8_wgrad(a, b, out32, offs.cuda(), True)
         _check(out32.cpu().double() - old32.double(), ref, "wgrad fp32 accumulate")
+
+
+def test_k_grouped_wgrad_on_column_slices_of_the_scale_array():
+    """The weight gradient of one half of a fused projection: rows of the transposed bytes (contiguous)
+    and a column slice of the scale array (its row stride is passed to the library)."""
+    from pith_train_amd.operators.grouped_linear import k_grouped_fp8_wgrad
+
+    sizes, N, K = [300, 0, 200, 128], 256, 128
+    ks, offs = _groups(sizes)
+    M, Gn = int(offs[-1]), len(sizes)
+    dy, x = _rand((M, N), 31), _rand((M, K), 32)
+    _, _, dy_ch, dy_s = Q.fp8cast_rowwise_colwise(dy)
+    _, _, x_ch, x_s = Q.fp8cast_rowwise_colwise(x)
+    tr = lambda q: q.view(torch.uint8).T.contiguous().view(torch.float8_e4m3fn).cuda()  # noqa: E731
+    dy_t, dy_sc, x_t, x_sc = tr(dy_ch), dy_s.cuda(), tr(x_ch), x_s.cuda()
+    half = N // 2
+    for lo in (0, half):
+        ref = G.gemm_k_grouped_wgrad(dy_ch[:, lo : lo + half].contiguous(), dy_s[:, lo : lo + half].contiguous(), x_ch, x_s,
+                                     offs, Gn, torch.float64).double()
+        out = torch.full((Gn, half, K), float("nan"), dtype=torch.bfloat16, device="cuda")
+        k_grouped_fp8_wgrad((dy_t[lo : lo + half], dy_sc[:, lo : lo + half]), (x_t, x_sc), out, offs.cuda(), False)
+        _check(out, ref, f"wgrad on scale columns {lo}..{lo + half}")

@@ -180,3 +180,15 @@ def test_row_limit_from_device_offsets_leaves_the_tail_untouched():
     assert torch.equal(ch_t[:, :real], u8(ref[2])) and torch.equal(ch_s[: real // 128], ref[3])
     assert (tok[real:] == 0x55).all() and (tok_s[real:] == -7.0).all()
     assert (ch_t[:, real:] == 0x55).all() and (ch_s[real // 128 :] == -7.0).all()
+
+
+def test_weights_quantised_into_a_fused_operand_equal_the_quantised_concatenation():
+    from pith_train_amd.operators import deepgemm_quantize as DQ
+
+    g = torch.Generator().manual_seed(21)
+    parts = [(torch.randn((3, n, 320), generator=g) * 0.02).bfloat16().cuda() for n in (128, 256, 128)]
+    got = DQ.fp8cast_blockwise_transpose_batched_cat(parts)
+    ref = DQ.fp8cast_blockwise_transpose_batched(torch.cat(parts, dim=1))
+    for a, b in zip(got, ref):
+        assert a.shape == b.shape
+        assert torch.equal(a.view(torch.uint8) if a.dtype != torch.float32 else a, b.view(torch.uint8) if b.dtype != torch.float32 else b)
