@@ -207,7 +207,7 @@ class GemmTimer:
         return rep
 
 
-def hbm_kernel_report(H, I, E, rows, eidx, top_k=8):
+def hbm_kernel_report(H, I, E, rows, eidx, top_k=8, kind="fused", extras=None):
     """HIP-event timings of the HBM-bound kernels of the path at this workload's shapes, called
     through the operator layer one at a time: achieved GB/s = algorithmic bytes (2 B per bf16,
     1 B per fp8 element, 4 B per 128-element scale) / time, against the 8 TB/s HBM peak."""
@@ -278,6 +278,51 @@ def hbm_kernel_report(H, I, E, rows, eidx, top_k=8):
     o = moe_combine(srcg, twg, res)
     rep("moe_combine_bwd_kernel [T,k,H]", timeit(lambda: torch.autograd.grad(o, [srcg, twg], res, retain_graph=True)),
         (2 * rows + T) * H * 2 + 8 * rows)
+    del srcg, twg, o, res, tw
+    extras = extras or {}
+    if kind == "gpt_oss":
+        # the epilogues of the GPT-OSS experts: interleaved gate/up with biases and the clamped SwiGLU
+        from pith_train_amd.operators.clamped_swiglu import clamped_swiglu
+        from pith_train_amd.operators.indexed_bias_add import indexed_bias_add
+        from pith_train_amd.operators.token_scatter import group_indices
+
+        gu = torch.randn((Mp, 2 * I), device="cuda", generator=g).bfloat16().requires_grad_(True)
+        bias = (torch.randn((E, 2 * I), device="cuda", generator=g) * 0.02).bfloat16().requires_grad_(True)
+        gids = group_indices(offs, Mp, torch.int64)
+        rep("bias_add_kernel (indexed_bias_add fwd) [Mp,2I]", timeit(lambda: indexed_bias_add(gu, bias, gids, offs)),
+            Mp * 2 * I * 4 + E * 2 * I * 2)
+        ob = indexed_bias_add(gu, bias, gids, offs)
+        dgu = torch.randn((Mp, 2 * I), device="cuda", generator=g).bfloat16()
+        rep("segment_sum_kernel (indexed_bias_add bwd: bias gradient) [Mp,2I]",
+            timeit(lambda: torch.autograd.grad(ob, bias, dgu, retain_graph=True)), Mp * 2 * I * 2 + E * 2 * I * 4)
+        del ob
+        rep("clamped_swiglu_fwd_kernel [Mp,I]", timeit(lambda: clamped_swiglu(gu, 1.702, 7.0)), Mp * I * 6)
+        oc = clamped_swiglu(gu, 1.702, 7.0)
+        dhh = torch.randn((Mp, I), device="cuda", generator=g).bfloat16()
+        rep("clamped_swiglu_bwd_kernel [Mp,I]", timeit(lambda: torch.autograd.grad(oc, gu, dhh, retain_graph=True)), Mp * I * 10)
+        del gu, bias, oc, dhh, dgu
+    if extras.get("dense_linears") or extras.get("shared_mlp"):
+        # quantisation kernels of the dense FP8 linears (activation / gradient / weight flavours)
+        T = rows // top_k
+        fin, fout = extras["dense_linears"][0] if extras.get("dense_linears") else (H, extras["shared_mlp"])
+        xa = torch.randn((T, fin), device="cuda", generator=g).bfloat16()
+        ga = torch.randn((T, fout), device="cuda", generator=g).bfloat16()
+        wa = (torch.randn((fout, fin), device="cuda", generator=g) * 0.02).bfloat16()
+        rep(f"quant_tile_kernel rowwise + 128x128 blockwise transpose (dense activations) [{T},{fin}]",
+            timeit(lambda: Q.fp8cast_rowwise_blockwise_transpose(xa)), T * fin * (4 + sc))
+        rep(f"quant_tile_kernel rowwise + rowwise of the transpose (dense gradients) [{T},{fout}]",
+            timeit(lambda: Q.fp8cast_rowwise_transpose(ga)), T * fout * (4 + 2 * sc))
+        rep(f"quant_tile_kernel 128x128 blockwise + transpose (dense weight) [{fout},{fin}]",
+            timeit(lambda: Q.fp8cast_blockwise_transpose(wa)), fout * fin * 4.0)
+    if "dedup_fraction" in extras:
+        # index construction of the dedup dispatch (integer only; bound by launch latency)
+        from pith_train_amd.operators import ep_dispatch as EP
+
+        T = rows // top_k
+        topk = make_routing(T, E, top_k, seed=5).cuda()
+        us = timeit(lambda: EP.fused_dedup_prepare_dispatch(topk, E, 8, E // 8))
+        out.append({"kernel": f"dd_* kernels (fused_dedup_prepare_dispatch, ep_size 8) [{T},{top_k}]", "us": round(us, 1),
+                    "algorithmic_MB": round(T * top_k * 8 * 4 / 1e6, 2), "note": "latency-bound chain of small integer kernels"})
     return out
 
 
@@ -483,7 +528,7 @@ def main():
         **extra,
     }
     if not args.no_kernel_report:
-        result["hbm_kernels"] = hbm_kernel_report(H, I, E, rows, eidx, k)
+        result["hbm_kernels"] = hbm_kernel_report(H, I, E, rows, eidx, k, kind, extras)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(kind, H, I, E, k, T, zipf)
         if extras:
