@@ -357,7 +357,7 @@ __global__ void group_indices_kernel(const int32_t* offs, int G, int64_t M, O* o
 // ---------------------------------------------------------------------------------------------
 // dedup dispatch
 // ---------------------------------------------------------------------------------------------
-static constexpr int kWaveTokens = 256;
+static constexpr int kWaveTokens = 64;  // tokens per wave of the dedup kernels (one step of 64 lanes)
 static constexpr int kMaxExperts = 1024;
 
 __device__ __forceinline__ int64_t topk_at(const int64_t* ids, int64_t ld, int k, int64_t flat) {
@@ -397,39 +397,72 @@ __global__ __launch_bounds__(256) void dd_hist_kernel(const int64_t* ids, int64_
   }
 }
 
-__global__ __launch_bounds__(1024) void dd_scan_kernel(int32_t* cnt_e, int32_t* cnt_g, int64_t W, int E, int ep, int epr,
-                                                       int64_t* tokens_per_ep_rank, int64_t* dedup_tokens_per_gpu,
-                                                       int64_t* send_meta, int32_t* expert_starts, int32_t* gpu_starts) {
-  __shared__ int32_t s_e[kMaxExperts];
-  __shared__ int32_t s_g[32];
-  for (int e = threadIdx.x; e < E; e += blockDim.x) {
-    int32_t run = 0;
-    for (int64_t w = 0; w < W; ++w) { const int32_t c = cnt_e[w * E + e]; cnt_e[w * E + e] = run; run += c; }
-    s_e[e] = run;
-  }
-  for (int g = threadIdx.x; g < ep; g += blockDim.x) {
-    int32_t run = 0;
-    for (int64_t w = 0; w < W; ++w) { const int32_t c = cnt_g[w * ep + g]; cnt_g[w * ep + g] = run; run += c; }
-    s_g[g] = run;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int32_t erun = 0, grun = 0;
-    for (int g = 0; g < ep; ++g) {
-      int64_t rank_total = 0;
-      for (int e = 0; e < epr; ++e) {
-        const int32_t c = s_e[g * epr + e];
-        expert_starts[g * epr + e] = erun;
-        erun += c;
-        rank_total += c;
-        send_meta[g * (epr + 1) + e] = c;
-      }
-      tokens_per_ep_rank[g] = rank_total;
-      dedup_tokens_per_gpu[g] = s_g[g];
-      gpu_starts[g] = grun;
-      grun += s_g[g];
-      send_meta[g * (epr + 1) + epr] = s_g[g];
+// Exclusive scan down one column of the per-wave count tables (column c < E: expert c, else EP rank
+// c - E), one wave per column, 64 chunks per step; the column total goes to totals[c].
+__global__ __launch_bounds__(256) void dd_scan_cols_kernel(int32_t* cnt_e, int32_t* cnt_g, int64_t W, int E, int ep,
+                                                           int32_t* totals /*[E + ep]*/) {
+  const int lane = threadIdx.x & 63;
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (c >= E + ep) return;
+  int32_t* col = c < E ? cnt_e + c : cnt_g + (c - E);
+  const int64_t stride = c < E ? E : ep;
+  int32_t run = 0;
+  for (int64_t w0 = 0; w0 < W; w0 += 64) {
+    const int64_t w = w0 + lane;
+    const int32_t v = w < W ? col[w * stride] : 0;
+    int32_t incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int32_t y = __shfl_up(incl, d);
+      if (lane >= d) incl += y;
     }
+    if (w < W) col[w * stride] = run + incl - v;
+    run += __shfl(incl, 63);
+  }
+  if (lane == 0) totals[c] = run;
+}
+
+// Starts of the experts and of the EP ranks from the column totals, and the per-rank metadata.
+__global__ __launch_bounds__(64) void dd_scan_totals_kernel(const int32_t* totals, int E, int ep, int epr,
+                                                            int64_t* tokens_per_ep_rank, int64_t* dedup_tokens_per_gpu,
+                                                            int64_t* send_meta, int32_t* expert_starts, int32_t* gpu_starts) {
+  const int lane = threadIdx.x;  // one wave
+  // exclusive scan over the experts, 64 at a time
+  int32_t run = 0;
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    const int e = e0 + lane;
+    const int32_t c = e < E ? totals[e] : 0;
+    int32_t incl = c;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int32_t y = __shfl_up(incl, d);
+      if (lane >= d) incl += y;
+    }
+    if (e < E) {
+      expert_starts[e] = run + incl - c;
+      send_meta[(e / epr) * (epr + 1) + (e % epr)] = c;
+    }
+    run += __shfl(incl, 63);
+  }
+  // per EP rank: rows routed to it, unique tokens sent to it, start of its slice of the dispatch list
+  const int g = lane;
+  int32_t sg = 0;
+  int64_t rank_total = 0;
+  if (g < ep) {
+    sg = totals[E + g];
+    for (int e = 0; e < epr; ++e) rank_total += totals[g * epr + e];
+  }
+  int32_t incl = sg;
+#pragma unroll
+  for (int d = 1; d < 32; d <<= 1) {
+    const int32_t y = __shfl_up(incl, d);
+    if (lane >= d) incl += y;
+  }
+  if (g < ep) {
+    tokens_per_ep_rank[g] = rank_total;
+    dedup_tokens_per_gpu[g] = sg;
+    gpu_starts[g] = incl - sg;
+    send_meta[g * (epr + 1) + epr] = sg;
   }
 }
 
@@ -666,7 +699,8 @@ extern "C" int pt_group_indices(const int32_t* offs, int32_t G, int64_t M, void*
 extern "C" int64_t pt_dedup_workspace_bytes(int64_t m, int32_t k, int32_t E, int32_t ep) {
   (void)k;
   const int64_t W = cdiv(m > 0 ? m : 1, kWaveTokens);
-  return align_up(W * E * 4, 256) + align_up(W * ep * 4, 256) + align_up((int64_t)E * 4, 256) + 256;
+  return align_up(W * E * 4, 256) + align_up(W * ep * 4, 256) + align_up((int64_t)E * 4, 256) + 256 +
+         align_up((int64_t)(E + ep) * 4, 256);
 }
 
 extern "C" int pt_dedup_prepare_dispatch(const int64_t* topk_ids, int64_t ld_ids, int64_t m, int32_t k, int32_t E,
@@ -685,11 +719,13 @@ extern "C" int pt_dedup_prepare_dispatch(const int64_t* topk_ids, int64_t ld_ids
   int32_t* cnt_e = (int32_t*)wsp; wsp += align_up(W * E * 4, 256);
   int32_t* cnt_g = (int32_t*)wsp; wsp += align_up(W * ep * 4, 256);
   int32_t* expert_starts = (int32_t*)wsp; wsp += align_up((int64_t)E * 4, 256);
-  int32_t* gpu_starts = (int32_t*)wsp;
+  int32_t* gpu_starts = (int32_t*)wsp; wsp += 256;
+  int32_t* totals = (int32_t*)wsp;
   const unsigned blocks = (unsigned)cdiv(W, 4);
   dd_hist_kernel<<<blocks, 256, (size_t)4 * (E + 32) * 4, s>>>(topk_ids, ld_ids, m, k, E, ep, epr, cnt_e, cnt_g);
-  dd_scan_kernel<<<1, 1024, 0, s>>>(cnt_e, cnt_g, W, E, ep, epr, tokens_per_ep_rank, dedup_tokens_per_gpu, send_meta,
-                                    expert_starts, gpu_starts);
+  dd_scan_cols_kernel<<<(unsigned)cdiv(E + ep, 4), 256, 0, s>>>(cnt_e, cnt_g, W, E, ep, totals);
+  dd_scan_totals_kernel<<<1, 64, 0, s>>>(totals, E, ep, epr, tokens_per_ep_rank, dedup_tokens_per_gpu, send_meta, expert_starts,
+                                         gpu_starts);
   const size_t lds = (size_t)4 * (E + 32 + 64 * ep) * 4;
   dd_rank_kernel<<<blocks, 256, lds, s>>>(topk_ids, ld_ids, m, k, E, ep, epr, bits_for(E), cnt_e, cnt_g, expert_starts,
                                           gpu_starts, dispatch_token_idxs, idxs, expand_idx);
