@@ -25,11 +25,14 @@ class FP8WeightCacheControl:
 
     @classmethod
     def clear(cls, *modules: nn.Module) -> None:
-        """Drop cached FP8 weights (``_wq_cache``) of every submodule to free memory."""
+        """Drop cached FP8 weights (``_wq_cache``, and the fused gate/up operand ``_gu_cache`` of
+        expert blocks with separate projections) of every submodule to free memory."""
         for root in modules:
             for m in root.modules():
                 if hasattr(m, "_wq_cache"):
                     m._wq_cache = None
+                if hasattr(m, "_gu_cache"):
+                    m._gu_cache = None
 
 
 class WeightGradStore:

@@ -42,6 +42,8 @@ class Qwen3MoeExperts(nn.Module):
         self.gate_proj = training.GroupedLinear(num_experts, hidden_size, moe_intermediate_size)
         self.up_proj = training.GroupedLinear(num_experts, hidden_size, moe_intermediate_size)
         self.down_proj = training.GroupedLinear(num_experts, moe_intermediate_size, hidden_size)
+        self._gu_cache = None  # gate and up quantised into one fused operand (FP8 path)
+        self._gu_version = -1
 
     def _fused_gate_up_quant(self):
         """gate and up weights quantised into one fused ``[G, 2I, H]`` operand; cached like the
@@ -50,7 +52,7 @@ class Qwen3MoeExperts(nn.Module):
         if torch.compiler.is_compiling():
             return fp8cast_blockwise_transpose_batched_cat(parts)
         ver = FP8WeightCacheControl.version
-        if getattr(self, "_gu_cache", None) is None or self._gu_version != ver:
+        if self._gu_cache is None or self._gu_version != ver:
             self._gu_cache = fp8cast_blockwise_transpose_batched_cat(parts)
             self._gu_version = ver
         return self._gu_cache
