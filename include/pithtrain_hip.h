@@ -145,6 +145,15 @@ int pt_gemm_m_grouped_nt_scatter(const void* a_fp8, const float* a_scale, const 
                                  int64_t K, const int32_t* out_row_index, int64_t out_rows,
                                  pt_stream_t stream);
 
+/* pt_gemm_m_grouped_nt followed by `out + bias[group of the row]` in the output type (the result
+ * is rounded to bf16, then the bias row of its group is added and the sum rounded again): the
+ * grouped linear and the indexed_bias_add after it (models/gpt_oss.py:151-156,
+ * indexed_bias_add.py:100-104) as one kernel.  bias is [G,N] bf16; N % 8 == 0. */
+int pt_gemm_m_grouped_nt_bias(const void* a_fp8, const float* a_scale, const void* b_fp8,
+                              const float* b_scale, void* out, int out_dtype, const int32_t* offs,
+                              int32_t num_groups, int64_t M, int64_t N, int64_t K,
+                              const void* bias, pt_stream_t stream);
+
 /* dW[g][n,k] = sum_{m in group g} dY[m,n] X[m,k] with colwise-quantised operands stored
  * transposed: dy_t[N,M] and x_t[K,M] (PT_CH_TRANSPOSED) and their scales dy_scale[M/128,N],
  * x_scale[M/128,K].  out is [G,N,K]:

@@ -37,6 +37,7 @@ SIGNATURES = {
                                                           I64, P]),
     "pt_gemm_nt_dense": (c_int, [P, P, P, P, P, c_int, I64, I64, I64, P]),
     "pt_gemm_m_grouped_nt": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P]),
+    "pt_gemm_m_grouped_nt_bias": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, P]),
     "pt_gemm_m_grouped_nt_scatter": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, I64, P]),
     "pt_gemm_k_grouped_wgrad": (c_int, [P, P, P, P, P, c_int, c_int, P, I32, I64, I64, I64, P]),
     "pt_gemm_k_grouped_wgrad_ld": (c_int, [P, P, I64, P, P, I64, P, c_int, c_int, P, I32, I64, I64, I64, P]),

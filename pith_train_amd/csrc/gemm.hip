@@ -304,7 +304,8 @@ static int dispatch_gemm(const GemmArgs& g, hipStream_t stream) {
   const int64_t lim = (1ll << 31) - 1;
   const bool fits = g.a_bytes < lim && g.b_bytes < lim && g.sa_bytes < lim && g.sb_bytes < lim && g.rows_a < lim &&
                     g.rows_b < lim && g.red < lim;
-  PT_REQUIRE(!g.out_row_index || (impl != IMPL_TILE && fits), "gemm: scattered output rows need the persistent kernel");
+  PT_REQUIRE((!g.out_row_index && !g.bias) || (impl != IMPL_TILE && fits),
+             "gemm: scattered output rows and the fused bias need the persistent kernels");
   if (impl == IMPL_TILE || !fits) return launch_gemm<128, 128, 2, 2>(g, stream);
   if (impl == IMPL_AUTO) return prefer_pipelined(g) ? launch_gemm_pipelined(g, 0, stream) : launch_gemm_persistent(g, 0, stream);
   if (impl >= IMPL_PIPELINED) return launch_gemm_pipelined(g, impl - IMPL_PIPELINED, stream);
@@ -346,7 +347,7 @@ extern "C" int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const v
 
 static int gemm_m_grouped_impl(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale, void* out,
                                int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N, int64_t K,
-                               const int32_t* out_row_index, int64_t out_rows, pt_stream_t stream) {
+                               const int32_t* out_row_index, int64_t out_rows, const void* bias, pt_stream_t stream) {
   PT_REQUIRE(M >= 0 && N >= 0 && K >= 0 && G > 0, "gemm_m_grouped_nt: bad sizes");
   if (M == 0 || N == 0) return PT_OK;
   PT_REQUIRE(M % 128 == 0, "gemm_m_grouped_nt: M=%lld must be a multiple of 128", (long long)M);
@@ -370,20 +371,33 @@ static int gemm_m_grouped_impl(const void* a_fp8, const float* a_scale, const vo
                "gemm_m_grouped_nt_scatter: needs N %% 8 == 0, a 16-byte aligned output smaller than 4 GiB");
     g.out_row_index = out_row_index; g.out_rows = out_rows;
   }
+  if (bias) {
+    PT_REQUIRE(!out_row_index && N % 8 == 0 && al16(out) && al16(bias),
+               "gemm_m_grouped_nt_bias: needs N %% 8 == 0 and 16-byte aligned output and bias, and no scattered rows");
+    g.bias = bias;
+  }
   return dispatch_gemm(g, (hipStream_t)stream);
 }
 
 extern "C" int pt_gemm_m_grouped_nt(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
                                     void* out, int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N, int64_t K,
                                     pt_stream_t stream) {
-  return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, nullptr, 0, stream);
+  return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, nullptr, 0, nullptr, stream);
 }
 
 extern "C" int pt_gemm_m_grouped_nt_scatter(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
                                             void* out, int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N,
                                             int64_t K, const int32_t* out_row_index, int64_t out_rows, pt_stream_t stream) {
   PT_REQUIRE(out_row_index, "gemm_m_grouped_nt_scatter: null out_row_index");
-  return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, out_row_index, out_rows, stream);
+  return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, out_row_index, out_rows, nullptr,
+                             stream);
+}
+
+extern "C" int pt_gemm_m_grouped_nt_bias(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
+                                         void* out, int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N,
+                                         int64_t K, const void* bias, pt_stream_t stream) {
+  PT_REQUIRE(bias, "gemm_m_grouped_nt_bias: null bias");
+  return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, nullptr, 0, bias, stream);
 }
 
 static int gemm_k_grouped_wgrad_impl(const void* dy_t_fp8, const float* dy_scale, int64_t ld_dy_scale, const void* x_t_fp8,

@@ -22,6 +22,7 @@ struct GemmArgs {
   int64_t total_tiles;
   const int32_t* out_row_index;           // m-grouped only: output row of result row r (negative: dropped); null = identity
   int64_t out_rows;                       // rows of the output when out_row_index is given
+  const void* bias;                       // m-grouped only: [G, rows_b] in the output's type, row g added to the rows of group g
 };
 
 

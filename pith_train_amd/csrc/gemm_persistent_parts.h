@@ -97,8 +97,11 @@ __device__ __forceinline__ void store_pairs_bf16(const v16f& a, __amdgpu_buffer_
 // need compiler fences only.
 // voff[q]: the lane's byte offset for tile rows 8q + lane/8, q = 0..3 (row start + 16-byte chunk
 // lane%8, or kOob); soff: uniform byte offset added to all of them.
+// bias (with has_bias): the 8 values of the lane's columns, added in the output type after the
+// result has been rounded to it (x + bias[group] as a second operation on the rounded x).
 __device__ __forceinline__ void store_staged_bf16_lines(const v16f& a0, const v16f& a1, __amdgpu_buffer_rsrc_t out, uint8_t* stg,
-                                                        const uint32_t (&voff)[4], uint32_t soff, bool accumulate, int lane) {
+                                                        const uint32_t (&voff)[4], uint32_t soff, bool accumulate, int lane,
+                                                        bool has_bias = false, v4i bias = v4i{0, 0, 0, 0}) {
   const bool odd = lane & 1;
   uint8_t* wr = stg + (4 * (lane >> 5) + (odd ? 1 : 0)) * 128 + ((lane & 31) >> 1) * 4;
   const uint8_t* rd = stg + (lane >> 3) * 128 + (lane & 7) * 16;
@@ -122,6 +125,11 @@ __device__ __forceinline__ void store_staged_bf16_lines(const v16f& a0, const v1
     for (int h = 0; h < 2; ++h) {
       v4i w = *(const v4i*)(rd + h * 1024);
       const uint32_t vo = voff[2 * hf + h];
+      if (has_bias) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          w[q] = (int)pack2_bf16(bf16_lo((uint32_t)w[q]) + bf16_lo((uint32_t)bias[q]), bf16_hi((uint32_t)w[q]) + bf16_hi((uint32_t)bias[q]));
+      }
       if (accumulate) {
         const v4i old = __builtin_amdgcn_raw_buffer_load_b128(out, vo, soff, 0);
 #pragma unroll
@@ -303,18 +311,22 @@ __device__ __forceinline__ void store_tile(v16f (&acc)[TM][TN], const GemmArgs& 
       }
     }
   } else if (p.out_dtype != PT_F32 && wide_ok && (T.b_lim & 7) == 0) {
+    const bool has_bias = MODE == GEMM_M_GROUPED && p.bias != nullptr;
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int j = 0; j < TN; j += 2) {
+      const int colc = T.b_row0 + wn0 + j * 32 + (lane & 7) * 8;
+      v4i bias = v4i{0, 0, 0, 0};
+      if (has_bias && colc < T.b_lim) bias = *(const v4i*)((const char*)p.bias + ((int64_t)T.g * p.rows_b + colc) * 2);
 #pragma unroll
-      for (int j = 0; j < TN; j += 2) {
-        const int colc = T.b_row0 + wn0 + j * 32 + (lane & 7) * 8;
+      for (int i = 0; i < TM; ++i) {
         uint32_t voff[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           voff[q] = colc < T.b_lim ? (uint32_t)(q * 8 + (lane >> 3)) * pitch + (uint32_t)(lane & 7) * 16 : kOob;
         if constexpr (PIN) { asm volatile("" : "+a"(acc[i][j])); asm volatile("" : "+a"(acc[i][j + 1])); }
-        store_staged_bf16_lines(acc[i][j], acc[i][j + 1], rs_out, stg, voff, s_tile + i * 32 * pitch + j * 64, ACC, lane);
+        store_staged_bf16_lines(acc[i][j], acc[i][j + 1], rs_out, stg, voff, s_tile + i * 32 * pitch + j * 64, ACC, lane, has_bias, bias);
       }
+    }
   } else if (p.out_dtype != PT_F32 && pair_ok && (T.b_lim & 1) == 0) {
     const bool odd = lane & 1;
 #pragma unroll

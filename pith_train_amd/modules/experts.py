@@ -154,21 +154,33 @@ class GptOssExperts(nn.Module):
             cache[name] = fp8cast_blockwise_transpose_batched(weight)
         return cache[name]
 
-    def _group_linear(self, x, weight, name, offs, ks, ks_tensor, group_indices_, in_rows=None):
+    def _group_linear(self, x, weight, name, offs, ks, ks_tensor, group_indices_, in_rows=None, bias=None):
         if x.shape[0] == 0:
             return x @ weight[0].transpose(-2, -1)
         if training.fp8:
             return FP8GroupedLinearFunc.apply(
-                x, weight, offs, ks, ks_tensor, self._quantized_weight(name, weight), group_indices_, in_rows
+                x, weight, offs, ks, ks_tensor, self._quantized_weight(name, weight), group_indices_, in_rows,
+                None, None, bias,
             )
         assert in_rows is None, "row maps need the FP8 layers"
         return GroupedLinearFunc.apply(x, weight, offs)
 
-    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None):
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None, fuse_bias: bool = True):
         """``row_map`` (extension, FP8 only): the scatter's int32 source-row map; ``x`` is then the
         un-permuted token tensor and the first quantisation gathers its rows (the result stays in
-        the grouped layout: the per-group bias gradients are sums over contiguous row ranges)."""
+        the grouped layout: the per-group bias gradients are sums over contiguous row ranges).
+        ``fuse_bias`` (FP8 only): the two ``indexed_bias_add`` steps happen in the stores of the
+        GEMMs before them (same bits)."""
         M = x.shape[0] if row_map is None else row_map.shape[0]
+        fused = (fuse_bias and training.fp8 and x.shape[0] > 0 and x.dtype == torch.bfloat16
+                 and self.gate_up_proj_bias.dtype == x.dtype and self.down_proj_bias.dtype == x.dtype
+                 and self.gate_up_proj.shape[1] % 8 == 0 and self.down_proj.shape[1] % 8 == 0)
+        if fused:
+            gate_up = self._group_linear(x, self.gate_up_proj, "gate_up_proj", grouped_mm_offs, ks, ks_tensor, None, row_map,
+                                         self.gate_up_proj_bias)
+            activated = clamped_swiglu(gate_up, 1.702, self.swiglu_limit)
+            return self._group_linear(activated, self.down_proj, "down_proj", grouped_mm_offs, ks, ks_tensor, None, None,
+                                      self.down_proj_bias)
         group_ids = group_indices(grouped_mm_offs, M, torch.int64)
         gate_up = self._group_linear(x, self.gate_up_proj, "gate_up_proj", grouped_mm_offs, ks, ks_tensor, None, row_map)
         gate_up = indexed_bias_add(gate_up, self.gate_up_proj_bias, group_ids, grouped_mm_offs)

@@ -106,14 +106,23 @@ class GroupedLinear(nn.Module):
 # FP8
 # ------------------------------------------------------------------------------------------------
 def m_grouped_fp8_gemm_nt(a, b, out: torch.Tensor, grouped_mm_offs: torch.Tensor,
-                          out_rows: torch.Tensor | None = None) -> torch.Tensor:
+                          out_rows: torch.Tensor | None = None, bias: torch.Tensor | None = None) -> torch.Tensor:
     """out[rows_g] = a[rows_g] @ b[g].T with a=(fp8[M,K], scale[M,K/128]), b=(fp8[G,N,K],
     scale[G,N/128,K/128]).  Rows at or past ``grouped_mm_offs[-1]`` are left untouched.  With
     ``out_rows`` (int32 [M]) result row r is written to ``out[out_rows[r]]`` instead (negative:
-    dropped)."""
+    dropped).  With ``bias`` ([G, N] in ``out``'s dtype) the bias row of a row's group is added
+    to the rounded result (``out + bias[group_ids]`` in the output dtype, as one kernel)."""
     (a_fp8, a_s), (b_fp8, b_s) = a, b
     M, K = a_fp8.shape
     G, N, _ = b_fp8.shape
+    if bias is not None:
+        assert out_rows is None and bias.shape == (G, N) and bias.dtype == out.dtype and bias.is_contiguous()
+        _lib.call(
+            "pt_gemm_m_grouped_nt_bias", a_fp8.data_ptr(), a_s.data_ptr(), b_fp8.data_ptr(), b_s.data_ptr(),
+            out.data_ptr(), _lib.dtype_code(out.dtype), grouped_mm_offs.data_ptr(), G, M, N, K, bias.data_ptr(),
+            _lib.stream_ptr(out.device),
+        )  # fmt: skip
+        return out
     if out_rows is not None:
         _lib.call(
             "pt_gemm_m_grouped_nt_scatter", a_fp8.data_ptr(), a_s.data_ptr(), b_fp8.data_ptr(),
@@ -206,8 +215,13 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
         in_rows: torch.Tensor | None = None,
         out_rows: torch.Tensor | None = None,
         out_m: int | None = None,
+        bias: torch.Tensor | None = None,
     ):
-        """``in_rows`` / ``out_rows`` (extension; int32 ``[M]`` source-row maps as produced by the
+        """``bias`` (extension; ``[G, N]`` in the input's dtype): ``indexed_bias_add`` of the result
+        folded into the GEMM's store (same bits as the two operators in a row; its gradient is the
+        per-group row sum of the incoming gradient).
+
+        ``in_rows`` / ``out_rows`` (extension; int32 ``[M]`` source-row maps as produced by the
         scatter, every non-negative value occurring once) fold the token permutation into this
         layer: with ``in_rows`` the input is the un-permuted ``[m, K]`` tensor and grouped row r is
         read from ``input[in_rows[r]]``; with ``out_rows`` the result is returned un-permuted
@@ -226,8 +240,10 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
         else:
             output = torch.empty((M, N), device=input.device, dtype=input.dtype)
         m_grouped_fp8_gemm_nt(
-            (input_fp8, scale_input), (weight_fp8, scale_weight), output, grouped_mm_offs, out_rows
+            (input_fp8, scale_input), (weight_fp8, scale_weight), output, grouped_mm_offs, out_rows,
+            bias.detach().contiguous() if bias is not None else None,
         )
+        ctx.bias_dtype = bias.dtype if bias is not None else None
         ctx.save_for_backward(
             weight_t_fp8, scale_weight_t, grouped_mm_offs, input_ch_t, scale_input_ch, ks_tensor,
             in_rows, out_rows,
@@ -257,7 +273,12 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
         )
 
         schedule_wgrad(weight, (grad_ch_t, scale_grad_ch), (input_ch_t, scale_input_ch), offs)
-        return grad_input, None, None, None, None, None, None, None, None, None
+        grad_bias = None
+        if ctx.bias_dtype is not None:
+            from .indexed_bias_add import _segment_sum_along_rows
+
+            grad_bias = _segment_sum_along_rows(grad_output, offs, ctx.bias_dtype)
+        return grad_input, None, None, None, None, None, None, None, None, None, grad_bias
 
 
 class FP8GroupedLinear(nn.Module):

@@ -125,3 +125,14 @@ def test_bench_refuses_more_than_one_gpu():
 
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_bench_times_every_gemm_entry_point_of_the_library():
+    """The roofline figure is only valid if no GEMM launch escapes the timer."""
+    import re
+
+    import bench
+
+    header = open(os.path.join(os.path.dirname(__file__), "..", "include", "pithtrain_hip.h")).read()
+    declared = set(re.findall(r"\bint (pt_gemm_(?!select_kernel)\w+)\(", header))
+    assert declared == set(bench.GemmTimer.NAMES), declared ^ set(bench.GemmTimer.NAMES)

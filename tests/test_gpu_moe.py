@@ -279,3 +279,32 @@ def test_dense_mlp_and_bf16_switch():
         assert training.Linear is torch.nn.Linear and training.GroupedLinear.__name__ == "GroupedLinear"
     finally:
         training.setup(True)
+
+
+@pytest.mark.parametrize("kind,E,H,I,T,k,zipf", [c for c in CASES if c[0] == "gpt_oss"] + [("gpt_oss", 8, 512, 256, 900, 4, 1.2)])
+def test_gpt_oss_bias_folded_into_the_gemm_store_is_bit_identical(kind, E, H, I, T, k, zipf):
+    """indexed_bias_add done by the store of the GEMM before it: same output, same token, weight
+    and bias gradients as the separate operator."""
+    import functools
+
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules.experts import forward_stage3
+
+    ids = OM.make_routing(T, E, k, seed=6, zipf_s=zipf)
+    g = torch.Generator().manual_seed(7)
+    tokens = torch.randn((T * k, H), generator=g).bfloat16().cuda()
+    dy = torch.randn((T * k, H), generator=g).bfloat16().cuda()
+    w = _weights(kind, E, H, I, 8)
+    res = []
+    for fuse_bias in (True, False):
+        mod, params = _build(kind, E, H, I, w)
+        mod.forward = functools.partial(mod.forward, fuse_bias=fuse_bias)
+        FP8WeightCacheControl.step()
+        tok = tokens.clone().requires_grad_(True)
+        out = forward_stage3(mod, tok, ids.reshape(-1).cuda(), E)
+        out.backward(dy)
+        res.append((out.detach(), tok.grad, {n: p.grad for n, p in params.items()}))
+    assert torch.equal(res[0][0], res[1][0]), "forward output differs"
+    assert torch.equal(res[0][1], res[1][1]), "token gradient differs"
+    for n in res[0][2]:
+        assert torch.equal(res[0][2][n], res[1][2][n]), f"{n} gradient differs"
