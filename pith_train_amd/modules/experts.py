@@ -57,10 +57,13 @@ class Qwen3MoeExperts(nn.Module):
             self._gu_version = ver
         return self._gu_cache
 
-    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None, fuse_activation: bool = True):
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None, fuse_activation: bool = True,
+                expand_idx=None):
         """``row_map`` (extension, FP8 layers only): the scatter's int32 source-row map.  ``x`` is
         then the un-permuted ``[m, H]`` token tensor and the result comes back un-permuted; the
-        permutation happens inside the first quantisation and the last GEMM's store.  With
+        permutation happens inside the first quantisation and the last GEMM's store.
+        ``expand_idx`` (one-node path only): ``x`` holds deduplicated rows, see
+        :func:`fused_experts.compose_row_maps`.  With
         ``fuse_activation`` (FP8 layers, intermediate size a multiple of 128) the block runs as one
         autograd node on a fused gate_up operand: the tokens are quantised once instead of once
         per projection, one GEMM serves both, and the SwiGLU and its gradient are computed inside
@@ -70,8 +73,9 @@ class Qwen3MoeExperts(nn.Module):
                 and fused_experts.supported_split(x, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight)):
             return fused_experts.FP8SwiGLUSplitExpertsFunc.apply(
                 x, self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight, grouped_mm_offs,
-                self._fused_gate_up_quant(), self.down_proj._get_quantized_weight(), row_map,
+                self._fused_gate_up_quant(), self.down_proj._get_quantized_weight(), row_map, expand_idx,
             )  # fmt: skip
+        assert expand_idx is None, "expand_idx needs the one-node FP8 path"
         gi = precompute_group_indices(grouped_mm_offs, x.shape[0])
         kwargs = dict(grouped_mm_offs=grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, group_indices=gi)
         if row_map is not None:
@@ -109,8 +113,9 @@ class Qwen35MoeExperts(nn.Module):
         self.gate_up_proj = training.GroupedLinear(num_experts, hidden_size, 2 * moe_intermediate_size)
         self.down_proj = training.GroupedLinear(num_experts, moe_intermediate_size, hidden_size)
 
-    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None, fuse_activation: bool = True):
-        """``row_map``: see :meth:`Qwen3MoeExperts.forward`.  With ``fuse_activation`` (FP8 layers)
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None, fuse_activation: bool = True,
+                expand_idx=None):
+        """``row_map`` / ``expand_idx``: see :meth:`Qwen3MoeExperts.forward`.  With ``fuse_activation`` (FP8 layers)
         the block runs as one autograd node whose SwiGLU output and SwiGLU gradient are computed
         inside the kernels that quantise them (same bits as the three-operator composition)."""
         if (fuse_activation and training.fp8 and x.shape[0] > 0 and isinstance(self.gate_up_proj, FP8GroupedLinear)
@@ -118,8 +123,9 @@ class Qwen35MoeExperts(nn.Module):
                 and fused_experts.supported(x, self.gate_up_proj.weight, self.down_proj.weight)):
             return fused_experts.FP8SwiGLUExpertsFunc.apply(
                 x, self.gate_up_proj.weight, self.down_proj.weight, grouped_mm_offs, ks, ks_tensor,
-                self.gate_up_proj._get_quantized_weight(), self.down_proj._get_quantized_weight(), row_map,
+                self.gate_up_proj._get_quantized_weight(), self.down_proj._get_quantized_weight(), row_map, expand_idx,
             )  # fmt: skip
+        assert expand_idx is None, "expand_idx needs the one-node FP8 path"
         gi = precompute_group_indices(grouped_mm_offs, x.shape[0])
         kwargs = dict(grouped_mm_offs=grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, group_indices=gi)
         if row_map is not None:
@@ -207,7 +213,7 @@ def forward_stage3(experts: nn.Module, gathered_tokens, expert_idxs, experts_per
     (each unique row is read once per use and no expanded copy is materialised); without it the
     two steps run separately as in the reference.
     """
-    if (fuse_permute and expand_idx is None and training.fp8 and expert_idxs.shape[0] > 0
+    if (fuse_permute and training.fp8 and expert_idxs.shape[0] > 0
             and isinstance(experts, (Qwen3MoeExperts, Qwen35MoeExperts))
             and isinstance(experts.down_proj, FP8GroupedLinear)
             and experts.down_proj.out_features % 8 == 0 and experts.down_proj.in_features % 8 == 0):
@@ -217,9 +223,15 @@ def forward_stage3(experts: nn.Module, gathered_tokens, expert_idxs, experts_per
             fused_node = (isinstance(experts.gate_proj, FP8GroupedLinear) and isinstance(experts.up_proj, FP8GroupedLinear)
                           and fused_experts.supported_split(gathered_tokens, experts.gate_proj.weight,
                                                             experts.up_proj.weight, experts.down_proj.weight))
-        _, grouped_mm_offs, ks, ks_tensor, src_of = group_rows_with_sizes(
-            expert_idxs, experts_per_rank, device=gathered_tokens.device, host_sizes=host_sizes or not fused_node)
-        return experts(gathered_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, row_map=src_of)
+        if expand_idx is None or (fused_node and fuse_expand):
+            _, grouped_mm_offs, ks, ks_tensor, src_of = group_rows_with_sizes(
+                expert_idxs, experts_per_rank, device=gathered_tokens.device, host_sizes=host_sizes or not fused_node)
+            if expand_idx is None:
+                return experts(gathered_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, row_map=src_of)
+            # deduplicated rows: the first quantisation reads them through expand_idx composed with
+            # the scatter's map, so neither the expanded nor the permuted copy exists
+            return experts(gathered_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, row_map=src_of,
+                           expand_idx=expand_idx)
     if (fuse_permute and expand_idx is None and training.fp8 and expert_idxs.shape[0] > 0
             and isinstance(experts, GptOssExperts)):
         # input side only: the output keeps the grouped layout for the per-group bias sums

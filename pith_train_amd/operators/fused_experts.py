@@ -71,31 +71,47 @@ def supported(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) ->
             and w_down.shape[1] % 8 == 0 and w_down.shape[2] == half)
 
 
-def _forward(ctx, x, gate_up_weights, w_down, grouped_mm_offs, q_gate_up, q_down, row_map):
+def compose_row_maps(row_map: torch.Tensor, expand_idx: torch.Tensor) -> torch.Tensor:
+    """``expand_idx[row_map]`` with the negative (padding) entries of ``row_map`` kept negative:
+    the source row of every grouped row when the routed rows are themselves an expansion
+    (``expand_idx``) of deduplicated rows."""
+    src = expand_idx[row_map.clamp(min=0).long()].to(torch.int32)
+    return torch.where(row_map >= 0, src, torch.full_like(src, -1))
+
+
+def _forward(ctx, x, gate_up_weights, w_down, grouped_mm_offs, q_gate_up, q_down, row_map, expand_idx=None):
     """Shared forward of the two autograd nodes below.  ``gate_up_weights``: the parameters whose
     gradients the gate_up weight gradient is written to, one fused ``[G, 2I, K]`` tensor or the
-    pair ``(gate [G, I, K], up [G, I, K])``."""
+    pair ``(gate [G, I, K], up [G, I, K])``.  ``expand_idx`` (with ``row_map``): ``x`` holds
+    deduplicated rows and routed row i is ``x[expand_idx[i]]``; the result has one row per routed
+    row, and the backward sums the gradients of the rows that share a source row."""
     _lib.require_cuda(x)
     gu_fp8, gu_scale, gu_t_fp8, gu_t_scale = q_gate_up
     dn_fp8, dn_scale, dn_t_fp8, dn_t_scale = q_down
     two_i = gu_fp8.shape[1]
     H = w_down.shape[1]
+    out_m = x.shape[0]
     if row_map is not None:
         M = row_map.shape[0]
-        x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, row_map, grouped_mm_offs)
+        in_map = row_map
+        if expand_idx is not None:
+            in_map = compose_row_maps(row_map, expand_idx)
+            out_m = expand_idx.shape[0]
+        x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, in_map, grouped_mm_offs)
     else:
+        assert expand_idx is None, "expand_idx needs the row map of the scatter"
         M = x.shape[0]
         x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t(x)
     gate_up = torch.empty((M, two_i), device=x.device, dtype=x.dtype)
     m_grouped_fp8_gemm_nt((x_fp8, x_s), (gu_fp8, gu_scale), gate_up, grouped_mm_offs)
     del x_fp8, x_s
     h_fp8, h_s, h_ch_t, h_ch_s = silu_mul_quant(gate_up, grouped_mm_offs if row_map is not None else None)
-    out = torch.empty((x.shape[0], H), device=x.device, dtype=x.dtype)
+    out = torch.empty((out_m, H), device=x.device, dtype=x.dtype)
     m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, row_map)
     ctx.save_for_backward(gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, grouped_mm_offs, x_ch_t, x_ch_s,
-                          gate_up, h_ch_t, h_ch_s, row_map)
+                          gate_up, h_ch_t, h_ch_s, row_map, expand_idx)
     ctx.gate_up_weights, ctx.w_down = gate_up_weights, w_down
-    ctx.rows = (M, x.shape[0])
+    ctx.rows = (M, out_m, x.shape[0])
     return out
 
 
@@ -103,8 +119,8 @@ def _backward(ctx, grad_out):
     """Shared backward: returns the gradient of ``x``; the weight gradients go to ``.grad`` (or to
     the ``WeightGradStore`` queue) through :func:`schedule_wgrad`."""
     (gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, offs, x_ch_t, x_ch_s, gate_up, h_ch_t, h_ch_s,
-     row_map) = ctx.saved_tensors  # fmt: skip
-    M, rows_x = ctx.rows
+     row_map, expand_idx) = ctx.saved_tensors  # fmt: skip
+    M, rows_x, rows_src = ctx.rows
     half = gate_up.shape[1] // 2
     K = gu_t_fp8.shape[1]
     grad_out = grad_out.contiguous()
@@ -119,6 +135,12 @@ def _backward(ctx, grad_out):
     dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s = silu_mul_bwd_quant(grad_h, gate_up, offs if row_map is not None else None)
     grad_x = torch.empty((rows_x, K), device=grad_out.device, dtype=grad_out.dtype)
     m_grouped_fp8_gemm_nt((dgu_fp8, dgu_s), (gu_t_fp8, gu_t_scale), grad_x, offs, row_map)
+    if expand_idx is not None:
+        # one gradient row per routed row so far: rows that expand the same source row are summed
+        # (the backward of the expanding gather, token_scatter.py:311-325)
+        from .token_scatter import _PaddedIndexGather
+
+        grad_x = _PaddedIndexGather.scatter_sum(grad_x, expand_idx, rows_src, 1024)
     if isinstance(ctx.gate_up_weights, tuple):
         # separate gate and up parameters: each gets the weight-gradient GEMM of its half of the
         # colwise twin (rows of the transposed bytes, columns of the scale array)
@@ -132,16 +154,16 @@ def _backward(ctx, grad_out):
 
 class FP8SwiGLUExpertsFunc(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w_gate_up, w_down, grouped_mm_offs, ks, ks_tensor, q_gate_up, q_down, row_map=None):
+    def forward(ctx, x, w_gate_up, w_down, grouped_mm_offs, ks, ks_tensor, q_gate_up, q_down, row_map=None, expand_idx=None):
         """``x`` is ``[M, K]`` grouped rows, or with ``row_map`` (int32 ``[M]``) the un-permuted
         ``[m, K]`` tokens; the result has the same row layout as ``x``.  ``row_map`` may be longer
         than the grouped rows (its tail negative): every kernel takes the real row count from
         ``grouped_mm_offs`` on the device, so no host-side size is needed (``ks`` may be None)."""
-        return _forward(ctx, x, w_gate_up, w_down, grouped_mm_offs, q_gate_up, q_down, row_map)
+        return _forward(ctx, x, w_gate_up, w_down, grouped_mm_offs, q_gate_up, q_down, row_map, expand_idx)
 
     @staticmethod
     def backward(ctx, grad_out):
-        return _backward(ctx, grad_out), None, None, None, None, None, None, None, None
+        return _backward(ctx, grad_out), None, None, None, None, None, None, None, None, None
 
 
 class FP8SwiGLUSplitExpertsFunc(torch.autograd.Function):
@@ -152,12 +174,12 @@ class FP8SwiGLUSplitExpertsFunc(torch.autograd.Function):
     gradients are written to the two parameters separately."""
 
     @staticmethod
-    def forward(ctx, x, w_gate, w_up, w_down, grouped_mm_offs, q_gate_up, q_down, row_map=None):
-        return _forward(ctx, x, (w_gate, w_up), w_down, grouped_mm_offs, q_gate_up, q_down, row_map)
+    def forward(ctx, x, w_gate, w_up, w_down, grouped_mm_offs, q_gate_up, q_down, row_map=None, expand_idx=None):
+        return _forward(ctx, x, (w_gate, w_up), w_down, grouped_mm_offs, q_gate_up, q_down, row_map, expand_idx)
 
     @staticmethod
     def backward(ctx, grad_out):
-        return _backward(ctx, grad_out), None, None, None, None, None, None, None
+        return _backward(ctx, grad_out), None, None, None, None, None, None, None, None
 
 
 def supported_split(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> bool:

@@ -136,7 +136,12 @@ def test_stage3_permute_folded_into_quant_and_gemm_is_bit_identical(kind, E, H, 
             assert ((a - b).abs() <= 2.0**-6 * b.abs().amax(dim=1, keepdim=True)).all(), "token gradient differs"
 
 
-def test_stage3_with_dedup_expand_fused_and_unfused():
+@pytest.mark.parametrize("kind", ["split", "fused"])
+def test_stage3_with_dedup_expand_fused_and_unfused(kind):
+    """Deduplicated rows (EP > 1): the path that reads them through ``expand_idx`` composed with
+    the scatter's map inside the first quantisation (no expanded and no permuted copy), the
+    expand folded into the scatter's row copy, and the reference's separate gather all agree
+    bit for bit, and with the oracle within the GEMM tolerance."""
     from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
     from pith_train_amd.modules.experts import forward_stage3
 
@@ -146,21 +151,26 @@ def test_stage3_with_dedup_expand_fused_and_unfused():
     expand = torch.randint(0, U, (R,), generator=g)
     eidx = torch.randint(0, E, (R,), generator=g)
     dy = torch.randn((R, H), generator=g).bfloat16()
-    w = _weights("split", E, H, I, 3)
-    ref = OM.moe_layer_fwd_bwd(uniq, eidx, w, dy, E, kind="split", fp8=True, expand_idx=expand, accum=torch.float64)
-    mod, params = _build("split", E, H, I, w)
-    grads = []
-    for fuse in (True, False):
+    w = _weights(kind, E, H, I, 3)
+    ref = OM.moe_layer_fwd_bwd(uniq, eidx, w, dy, E, kind=kind, fp8=True, expand_idx=expand, accum=torch.float64)
+    res = []
+    for fuse_permute, fuse_expand in ((True, True), (False, True), (False, False), (True, False)):
+        mod, params = _build(kind, E, H, I, w)
         FP8WeightCacheControl.step()
-        for p in params.values():
-            p.grad = None
         t = uniq.cuda().requires_grad_(True)
-        out = forward_stage3(mod, t, eidx.cuda(), E, expand_idx=expand.cuda(), fuse_expand=fuse)
-        _close(out, ref["out"], f"out fuse={fuse}")
+        out = forward_stage3(mod, t, eidx.cuda(), E, expand_idx=expand.cuda(), fuse_expand=fuse_expand,
+                             fuse_permute=fuse_permute)
+        assert out.shape == (R, H)
+        _close(out, ref["out"], f"out permute={fuse_permute} expand={fuse_expand}")
         out.backward(dy.cuda())
-        _close(t.grad, ref["grad_tokens"], f"grad_tokens fuse={fuse}")
-        grads.append(t.grad.clone())
-    assert torch.equal(grads[0], grads[1])
+        assert t.grad.shape == (U, H)
+        _close(t.grad, ref["grad_tokens"], f"grad_tokens permute={fuse_permute} expand={fuse_expand}")
+        res.append((out.detach(), t.grad.clone(), {n: p.grad for n, p in params.items()}))
+    for other in res[1:]:
+        assert torch.equal(res[0][0], other[0]), "forward output differs"
+        assert torch.equal(res[0][1], other[1]), "token gradient differs"
+        for n in res[0][2]:
+            assert torch.equal(res[0][2][n], other[2][n]), f"{n} gradient differs"
 
 
 def test_grouped_linear_defers_wgrad_and_accumulates():
