@@ -279,7 +279,16 @@ def hbm_kernel_report(H, I, E, rows, eidx, top_k=8, kind="fused", extras=None):
     o = moe_combine(srcg, twg, res)
     rep("moe_combine_bwd_kernel [T,k,H]", timeit(lambda: torch.autograd.grad(o, [srcg, twg], res, retain_graph=True)),
         (2 * rows + T) * H * 2 + 8 * rows)
-    del srcg, twg, o, res, tw
+    # the expert-parallel branch of the same step: rows arrive in the dispatch sort's order
+    from pith_train_amd.operators.moe_combine import moe_combine_ep
+
+    local_idxs = torch.argsort(eidx, stable=True)
+    rep("moe_combine_ep_fwd_kernel (+ slot index) [T,k,H]", timeit(lambda: moe_combine_ep(srcg, local_idxs, twg, res)),
+        (rows + 2 * T) * H * 2 + 20 * rows)
+    o = moe_combine_ep(srcg, local_idxs, twg, res)
+    rep("moe_combine_bwd_kernel, rows through the slot index [T,k,H]",
+        timeit(lambda: torch.autograd.grad(o, [srcg, twg], res, retain_graph=True)), (2 * rows + T) * H * 2 + 12 * rows)
+    del srcg, twg, o, res, tw, local_idxs
     extras = extras or {}
     if kind == "gpt_oss":
         # the epilogues of the GPT-OSS experts: interleaved gate/up with biases and the clamped SwiGLU

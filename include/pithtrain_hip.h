@@ -322,6 +322,29 @@ int pt_moe_combine_bwd(const void* grad_out, int64_t ld_go, const void* moe, int
                        const float* topk_weight, void* d_moe, int64_t ld_dmoe, float* d_weight,
                        int64_t T, int32_t k, int64_t H, int dtype, pt_stream_t stream);
 
+/* Expert-parallel branch of forward_stage5 (models/qwen3_moe.py:238-245, same lines in
+ * deepseek_v2.py:351-357, qwen35_moe.py:334-340, gpt_oss.py:334-340): row r of moe [rows,H] belongs
+ * to the flat top-k slot local_idxs[r] (token local_idxs[r] / k), every weighted row is rounded to
+ * S and added to a zeroed S accumulator, the residual is added last.  The reference's scatter_add_
+ * leaves the order of the adds to the device's atomics; here a token's rows are added in ascending
+ * r, every partial sum rounded to S (the result of a sequential scatter_add_).
+ *
+ * pt_moe_combine_ep_index: slot_row[s] = r for s = local_idxs[r], -1 for slots without a row
+ * (slot_row int32 [slots], slots = T*k; entries of local_idxs must be distinct, values outside
+ * [0, slots) are ignored). */
+int pt_moe_combine_ep_index(const int64_t* local_idxs, int64_t rows, int64_t slots,
+                            int32_t* slot_row, pt_stream_t stream);
+int pt_moe_combine_ep_fwd(const void* moe, int64_t ld_moe, int64_t rows, const int32_t* slot_row,
+                          const float* topk_weight, const void* residual, int64_t ld_res, void* out,
+                          int64_t ld_out, int64_t T, int32_t k, int64_t H, int dtype,
+                          pt_stream_t stream);
+/* d_moe[r,:] = S(float(grad_out[t,:]) * topk_weight[t,j]) for r = slot_row[t*k+j];
+ * d_weight[t,j] = sum_h grad_out[t,h] * moe[r,h] in fp32, 0 for a slot without a row. */
+int pt_moe_combine_ep_bwd(const void* grad_out, int64_t ld_go, const void* moe, int64_t ld_moe,
+                          int64_t rows, const int32_t* slot_row, const float* topk_weight,
+                          void* d_moe, int64_t ld_dmoe, float* d_weight, int64_t T, int32_t k,
+                          int64_t H, int dtype, pt_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
