@@ -289,6 +289,16 @@ def hbm_kernel_report(H, I, E, rows, eidx, top_k=8, kind="fused", extras=None):
     rep("moe_combine_bwd_kernel, rows through the slot index [T,k,H]",
         timeit(lambda: torch.autograd.grad(o, [srcg, twg], res, retain_graph=True)), (2 * rows + T) * H * 2 + 12 * rows)
     del srcg, twg, o, res, tw, local_idxs
+    # the step before the path: softmax / top-k / weights of the router gate (after its logits GEMM)
+    from pith_train_amd.operators.router_topk import softmax_topk, topk_softmax
+
+    lg = (torch.randn((T, E), device="cuda", generator=g) * 2).bfloat16().requires_grad_(True)
+    route = (lambda: topk_softmax(lg, top_k)) if kind == "gpt_oss" else (lambda: softmax_topk(lg, top_k, norm_topk_prob=True))
+    rep("router_topk_fwd_kernel [T,E] -> [T,k]", timeit(route), T * E * 2 + T * top_k * 12)
+    o = route()[1]
+    rep("router_topk_bwd_kernel [T,k] -> [T,E]", timeit(lambda: torch.autograd.grad(o, lg, o.detach(), retain_graph=True)),
+        2 * T * E * 2 + T * top_k * 12)
+    del lg, o
     extras = extras or {}
     if kind == "gpt_oss":
         # the epilogues of the GPT-OSS experts: interleaved gate/up with biases and the clamped SwiGLU

@@ -345,6 +345,33 @@ int pt_moe_combine_ep_bwd(const void* grad_out, int64_t ld_go, const void* moe, 
                           void* d_moe, int64_t ld_dmoe, float* d_weight, int64_t T, int32_t k,
                           int64_t H, int dtype, pt_stream_t stream);
 
+/* Router gate after the logits GEMM: softmax + top-k + weights of the chosen experts, one launch.
+ *   mode 0: Qwen3MoeGate.forward (models/qwen3_moe.py:81-88), Qwen35MoeTopKRouter.forward
+ *           (models/qwen35_moe.py:216-222) and DeepSeekV2MoEGate.forward (models/deepseek_v2.py:
+ *           149-164): scores = softmax(logits) in fp32; with num_group > 1 only the topk_group
+ *           groups of E/num_group contiguous experts with the largest maximum keep their scores
+ *           (group_limited_greedy), the rest become 0; top-k of the scores; w = scores[topk_idx];
+ *           w /= sum(w) if norm_topk_prob; w *= scale (routed_scaling_factor).
+ *   mode 1: GptOssTopKRouter.forward (models/gpt_oss.py:176-182): top-k of the logits, then
+ *           w = softmax(logits[topk_idx]) in fp32.
+ * logits [T,E] in dtype (leading dimension in elements), E <= 512, k <= min(32, E).  topk_idx int64
+ * [T,k] comes out sorted by descending value, ties to the lower expert index (torch.topk leaves
+ * both open for sorted=False).  forced_idx (router replay, the `router_replay` hook of the same
+ * functions) replaces the selection when not null.  scores fp32 [T,E] (what the load-balance loss
+ * reads: after the group limit in mode 0, the full softmax in mode 1) is written when not null. */
+int pt_router_topk_fwd(const void* logits, int64_t ld_logits, int dtype, int64_t T, int32_t E,
+                       int32_t k, int mode, int norm_topk_prob, float scale, int32_t num_group,
+                       int32_t topk_group, const int64_t* forced_idx, int64_t* topk_idx,
+                       float* topk_weight, float* scores, pt_stream_t stream);
+/* Gradient of the logits from d_weight fp32 [T,k] (and d_scores fp32 [T,E] when not null), through
+ * the scale, the normalisation, the gather at topk_idx, the group limit and the softmax; the
+ * scores are recomputed from the logits.  d_logits [T,E] in dtype. */
+int pt_router_topk_bwd(const void* logits, int64_t ld_logits, int dtype, int64_t T, int32_t E,
+                       int32_t k, int mode, int norm_topk_prob, float scale, int32_t num_group,
+                       int32_t topk_group, const int64_t* topk_idx, const float* d_weight,
+                       const float* d_scores, void* d_logits, int64_t ld_dlogits,
+                       pt_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
