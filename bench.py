@@ -299,6 +299,20 @@ def hbm_kernel_report(H, I, E, rows, eidx, top_k=8, kind="fused", extras=None):
     rep("router_topk_bwd_kernel [T,k] -> [T,E]", timeit(lambda: torch.autograd.grad(o, lg, o.detach(), retain_graph=True)),
         2 * T * E * 2 + T * top_k * 12)
     del lg, o
+    # the loss head: in-place fused cross-entropy over a 151 936-entry vocabulary (Qwen3), 4096 rows
+    from pith_train_amd import _lib
+    from pith_train_amd.operators.cross_entropy import cross_entropy
+
+    Nce, Vce = 4096, 151936
+    logits = (torch.randn((Nce, Vce), device="cuda", generator=g) * 2).bfloat16()
+    tgt = torch.randint(0, Vce, (Nce,), device="cuda", generator=g)
+    rep("ce_fwd_onchip_kernel (cross_entropy forward, in place) [N,V]", timeit(lambda: cross_entropy(logits, tgt)),
+        2 * Nce * Vce * 2)
+    half = torch.full((1,), 0.5, device="cuda")
+    rep("ce_scale_kernel (cross_entropy backward, in place) [N,V]",
+        timeit(lambda: _lib.call("pt_cross_entropy_bwd", logits.data_ptr(), Vce, _lib.dtype_code(logits.dtype), Nce, Vce,
+                                 half.data_ptr(), _lib.stream_ptr(logits.device))), 2 * Nce * Vce * 2)
+    del logits, tgt
     extras = extras or {}
     if kind == "gpt_oss":
         # the epilogues of the GPT-OSS experts: interleaved gate/up with biases and the clamped SwiGLU

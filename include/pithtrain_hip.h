@@ -372,6 +372,21 @@ int pt_router_topk_bwd(const void* logits, int64_t ld_logits, int dtype, int64_t
                        const float* d_scores, void* d_logits, int64_t ld_dlogits,
                        pt_stream_t stream);
 
+/* In-place fused cross-entropy with mean reduction (CrossEntropy.forward and its Triton kernel
+ * cross_entropy_fwd, operators/cross_entropy.py:16-78,86-118): logits [N,V] in dtype are
+ * overwritten with the gradient of the mean loss, S((exp(x - max) / sum) / n) and, at the target,
+ * S(float(stored) - 1/n), with n = max(1, number of rows whose target is not ignore_index); rows
+ * with the ignored target become zero.  loss_rows fp32 [N] receives -(x_y - max - log sum) (0 for
+ * ignored rows, NaN for a target outside [0, V)), loss fp32 [1] their sum over n, n_non_ignore
+ * int64 [1] n itself.  Three launches on the stream, no host synchronisation. */
+int pt_cross_entropy_fwd(void* logits, int64_t ld, int dtype, const int64_t* target, int64_t N,
+                         int64_t V, int64_t ignore_index, float* loss_rows, float* loss,
+                         int64_t* n_non_ignore, pt_stream_t stream);
+/* CrossEntropy.backward (operators/cross_entropy.py:120-124): the stored gradient times the
+ * incoming scalar (fp32 on the device, rounded to dtype first), in place. */
+int pt_cross_entropy_bwd(void* grad, int64_t ld, int dtype, int64_t N, int64_t V,
+                         const float* grad_output, pt_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
