@@ -234,6 +234,12 @@ int pt_gather_rows_backward(const void* grad_out, int64_t ld_go, void* grad_in, 
  * models/gpt_oss.py:146-150. */
 int pt_group_indices(const int32_t* offs, int32_t num_groups, int64_t M, void* group_ids,
                      int32_t out_dtype_bytes, pt_stream_t stream);
+/* out[r] = expand_idx[row_map[r]] (int32) where row_map[r] is in [0, n_expand) and the result in
+ * [0, n_src), -1 otherwise.  Composes the scatter's source map with the dedup expand index
+ * (models/qwen3_moe.py:222-224 gathers through expand_idx, then scatters), so that the first
+ * quantisation of the expert block reads the deduplicated rows directly. */
+int pt_compose_row_map(const int32_t* row_map, int64_t n, const int64_t* expand_idx,
+                       int64_t n_expand, int64_t n_src, int32_t* out, pt_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Expert-parallel dispatch index construction with token dedup.

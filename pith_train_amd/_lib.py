@@ -46,6 +46,7 @@ SIGNATURES = {
     "pt_moe_combine_bwd": (c_int, [P, I64, P, I64, P, P, I64, P, I64, I32, I64, c_int, P]),
     "pt_router_topk_fwd": (c_int, [P, I64, c_int, I64, I32, I32, c_int, c_int, F, I32, I32, P, P, P, P, P]),
     "pt_router_topk_bwd": (c_int, [P, I64, c_int, I64, I32, I32, c_int, c_int, F, I32, I32, P, P, P, P, I64, P]),
+    "pt_compose_row_map": (c_int, [P, I64, P, I64, I64, P, P]),
     "pt_probe_mfma_rate": (c_int, [I32, I32, P, P, P]),
     "pt_cross_entropy_fwd": (c_int, [P, I64, c_int, P, I64, I64, I64, P, P, P, P]),
     "pt_cross_entropy_bwd": (c_int, [P, I64, c_int, I64, I64, P, P]),

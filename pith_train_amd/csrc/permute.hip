@@ -696,6 +696,30 @@ extern "C" int pt_group_indices(const int32_t* offs, int32_t G, int64_t M, void*
   return check_launch("group_indices");
 }
 
+// out[r] = expand_idx[row_map[r]] for row_map[r] in [0, n_expand), -1 otherwise: the source row of
+// every grouped row when the routed rows are themselves an expansion of deduplicated rows.
+__global__ __launch_bounds__(256) void compose_row_map_kernel(const int32_t* row_map, int64_t n, const int64_t* expand_idx,
+                                                              int64_t n_expand, int64_t n_src, int32_t* out) {
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= n) return;
+  const int32_t i = row_map[r];
+  int64_t s = -1;
+  if (i >= 0 && i < n_expand) {
+    s = expand_idx[i];
+    if (s < 0 || s >= n_src) s = -1;  // an index outside the source rows reads nothing
+  }
+  out[r] = (int32_t)s;
+}
+
+extern "C" int pt_compose_row_map(const int32_t* row_map, int64_t n, const int64_t* expand_idx, int64_t n_expand,
+                                  int64_t n_src, int32_t* out, pt_stream_t stream) {
+  PT_REQUIRE(n >= 0 && n_expand >= 0 && n_src >= 0 && n_src < (1ll << 31), "compose_row_map: bad sizes");
+  if (n == 0) return PT_OK;
+  PT_REQUIRE(row_map && out && (expand_idx || n_expand == 0), "compose_row_map: null pointer");
+  compose_row_map_kernel<<<(unsigned)cdiv(n, 256), 256, 0, (hipStream_t)stream>>>(row_map, n, expand_idx, n_expand, n_src, out);
+  return check_launch("compose_row_map");
+}
+
 extern "C" int64_t pt_dedup_workspace_bytes(int64_t m, int32_t k, int32_t E, int32_t ep) {
   (void)k;
   const int64_t W = cdiv(m > 0 ? m : 1, kWaveTokens);

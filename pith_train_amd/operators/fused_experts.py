@@ -71,12 +71,17 @@ def supported(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) ->
             and w_down.shape[1] % 8 == 0 and w_down.shape[2] == half)
 
 
-def compose_row_maps(row_map: torch.Tensor, expand_idx: torch.Tensor) -> torch.Tensor:
+def compose_row_maps(row_map: torch.Tensor, expand_idx: torch.Tensor, n_src: int) -> torch.Tensor:
     """``expand_idx[row_map]`` with the negative (padding) entries of ``row_map`` kept negative:
-    the source row of every grouped row when the routed rows are themselves an expansion
-    (``expand_idx``) of deduplicated rows."""
-    src = expand_idx[row_map.clamp(min=0).long()].to(torch.int32)
-    return torch.where(row_map >= 0, src, torch.full_like(src, -1))
+    the source row (among ``n_src``) of every grouped row when the routed rows are themselves an
+    expansion (``expand_idx``) of deduplicated rows."""
+    assert row_map.dtype == torch.int32 and expand_idx.dtype == torch.int64
+    out = torch.empty_like(row_map)
+    _lib.call(
+        "pt_compose_row_map", row_map.contiguous().data_ptr(), row_map.numel(), expand_idx.contiguous().data_ptr(),
+        expand_idx.numel(), n_src, out.data_ptr(), _lib.stream_ptr(row_map.device),
+    )  # fmt: skip
+    return out
 
 
 def _forward(ctx, x, gate_up_weights, w_down, grouped_mm_offs, q_gate_up, q_down, row_map, expand_idx=None):
@@ -95,7 +100,7 @@ def _forward(ctx, x, gate_up_weights, w_down, grouped_mm_offs, q_gate_up, q_down
         M = row_map.shape[0]
         in_map = row_map
         if expand_idx is not None:
-            in_map = compose_row_maps(row_map, expand_idx)
+            in_map = compose_row_maps(row_map, expand_idx, x.shape[0])
             out_m = expand_idx.shape[0]
         x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, in_map, grouped_mm_offs)
     else:
