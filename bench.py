@@ -427,6 +427,9 @@ def main():
                     help="skip the extra (untimed-for-value) pass that keeps the FP8 weight cache across steps")
     ap.add_argument("--no-kernel-report", action="store_true",
                     help="skip the per-kernel GB/s table of the HBM-bound kernels (hbm_kernels in the JSON line)")
+    ap.add_argument("--kernel-report-only", action="store_true",
+                    help="run only the per-kernel table (what a `rocprofv3 --kernel-trace` of the HBM-bound "
+                         "kernels traces) and print it as the JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="after the timed region launch gather_rows_kernel as a plain copy of 256 MiB "
                          "(identity index) three times: the known-size kernel that FETCH_SIZE / "
@@ -461,6 +464,9 @@ def main():
         expand_idx = expand_cpu.cuda()
     else:
         tokens = x.cuda().unsqueeze(1).expand(-1, k, -1).reshape(-1, H).contiguous()
+    if args.kernel_report_only:
+        print(json.dumps({"workload": args.workload, "hbm_kernels": hbm_kernel_report(H, I, E, rows, eidx, k, kind, extras)}))
+        return
     flops = gemm_flops(rows, H, I) + extra_flops(extras, T, H)
     dense = []  # (module, input [T, in], upstream grad [T, out])
     if extras.get("shared_mlp") or extras.get("dense_linears"):

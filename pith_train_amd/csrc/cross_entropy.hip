@@ -177,8 +177,8 @@ __global__ __launch_bounds__(1024) void ce_fwd_kernel(CeArgs p) {
 // kCeRegChunks 16-byte chunks per thread in registers and the chunks past those in LDS, so the
 // logits cross the memory bus once each way (the generic kernel's second read of a 300 KB row
 // mostly misses the caches when 256 rows are in flight).
-static constexpr int kCeRegChunks = 16;                                  // 16 x 1024 x 8 = 131 072 elements
-static constexpr int kCeLdsChunks = 9 * 1024;                            // + 73 728 elements in 144 KiB of LDS
+static constexpr int kCeRegChunks = 15;                                  // 15 x 1024 x 8 = 122 880 elements
+static constexpr int kCeLdsChunks = (160 * 1024 - 256) / 16;             // + 81 792 elements in the rest of the 160 KiB of LDS
 
 typedef int ce_v4i __attribute__((ext_vector_type(4)));
 
@@ -186,6 +186,15 @@ template <typename S>
 __device__ __forceinline__ void unpack8(const ce_v4i& w, float* v) {
   static_assert(S::kBytes == 2, "16-bit storage only");
   S::load8(&w, v);
+}
+
+// 16 bytes per lane from base + voff (per lane) + soff (uniform) into LDS at lds_off + 16 * lane.
+__device__ __forceinline__ void ce_load_to_lds(ce_v4i rsrc, uint32_t voff, uint32_t soff, uint32_t lds_off) {
+  soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
+  lds_off = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_off);
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff),
+               "s"(lds_off)
+               : "memory");
 }
 
 template <typename S>
@@ -206,6 +215,14 @@ __global__ __launch_bounds__(1024) void ce_fwd_onchip_kernel(CeArgs p) {
   // chunk's i * 16 KiB goes into the uniform offset, and accesses past the row's end are dropped by
   // the hardware (loads return 0) instead of needing an address and a predicate per chunk.
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(x, 0, (int)(p.V * S::kBytes), 0x00020000);
+  ce_v4i rsrc_words;  // the same descriptor as plain words, for the inline-assembly load
+  {
+    const uint64_t a = (uint64_t)(uintptr_t)x;
+    rsrc_words[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+    rsrc_words[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((a >> 32) & 0xFFFF));
+    rsrc_words[2] = __builtin_amdgcn_readfirstlane((int)(p.V * S::kBytes));
+    rsrc_words[3] = 0x00020000;
+  }
   const uint32_t voff = (uint32_t)tid * 16u;
   ce_v4i cache[kCeRegChunks];
   float m = -INFINITY, d = 0.f;
@@ -228,16 +245,24 @@ __global__ __launch_bounds__(1024) void ce_fwd_onchip_kernel(CeArgs p) {
     }
     __builtin_amdgcn_sched_barrier(0);  // one chunk's temporaries at a time: the cache owns the registers
   };
+  // The chunks past the registers go straight from memory into LDS (direct-to-LDS loads: a wave's
+  // 64 lanes fill 1 KiB, lane l the 16 bytes of the chunk thread l of that wave owns), issued first
+  // so that they travel while the register part is loaded and absorbed.
+  {
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) ce_v4i*)s_over;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+#pragma unroll 1
+    for (uint32_t c0 = kCeRegChunks * kCeThreads + wave * 64; c0 < p.chunks; c0 += kCeThreads)
+      ce_load_to_lds(rsrc_words, (uint32_t)(tid & 63) * 16u, c0 * 16u, lds_base + (c0 - kCeRegChunks * kCeThreads) * 16u);
+  }
 #pragma unroll
   for (int i = 0; i < kCeRegChunks; ++i) cache[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kCeThreads * 16, 0);
 #pragma unroll
   for (int i = 0; i < kCeRegChunks; ++i)
     if ((uint32_t)i * kCeThreads + tid < p.chunks) absorb(cache[i]);
-  for (uint32_t c = kCeRegChunks * kCeThreads + tid; c < p.chunks; c += kCeThreads) {
-    const ce_v4i w = *(const ce_v4i*)(x + (int64_t)c * 16);
-    s_over[c - kCeRegChunks * kCeThreads] = w;  // read back by the same thread in pass 2
-    absorb(w);
-  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the LDS part has landed (each thread reads only its own chunks)
+#pragma unroll 1
+  for (uint32_t c = kCeRegChunks * kCeThreads + tid; c < p.chunks; c += kCeThreads) absorb(s_over[c - kCeRegChunks * kCeThreads]);
 #pragma unroll
   for (int s = 32; s >= 1; s >>= 1) {
     const float m2 = __shfl_xor(m, s), d2 = __shfl_xor(d, s);
@@ -285,6 +310,7 @@ __global__ __launch_bounds__(1024) void ce_fwd_onchip_kernel(CeArgs p) {
     __builtin_amdgcn_raw_buffer_store_b128(grad_of(cache[i], c), rsrc, voff, i * kCeThreads * 16, 0);
     __builtin_amdgcn_sched_barrier(0);
   }
+#pragma unroll 1
   for (uint32_t c = kCeRegChunks * kCeThreads + tid; c < p.chunks; c += kCeThreads)
     *(ce_v4i*)(x + (int64_t)c * 16) = grad_of(s_over[c - kCeRegChunks * kCeThreads], c);
 }
