@@ -213,3 +213,21 @@ def test_k_grouped_wgrad_on_column_slices_of_the_scale_array():
         out = torch.full((Gn, half, K), float("nan"), dtype=torch.bfloat16, device="cuda")
         k_grouped_fp8_wgrad((dy_t[lo : lo + half], dy_sc[:, lo : lo + half]), (x_t, x_sc), out, offs.cuda(), False)
         _check(out, ref, f"wgrad on scale columns {lo}..{lo + half}")
+
+
+def test_mfma_rate_probe_runs_and_counts_its_work():
+    """The measurement aid bench.py times: launches, fills its sink, reports 2 * 32 * 32 * 64 FLOP
+    per instruction x 8 per iteration x 4 waves per workgroup."""
+    import ctypes
+
+    from pith_train_amd import _lib
+
+    blocks, iters = 64, 10
+    sink = torch.full((blocks * 256,), float("nan"), device="cuda")
+    flop = ctypes.c_double()
+    _lib.call("pt_probe_mfma_rate", blocks, iters, sink.data_ptr(), ctypes.addressof(flop), _lib.stream_ptr(sink.device))
+    torch.cuda.synchronize()
+    assert flop.value == 2.0 * 32 * 32 * 64 * 8 * iters * 4 * blocks
+    assert not torch.isnan(sink).any()
+    with pytest.raises(_lib.PithTrainHipError):
+        _lib.call("pt_probe_mfma_rate", 0, iters, sink.data_ptr(), ctypes.addressof(flop), _lib.stream_ptr(sink.device))
