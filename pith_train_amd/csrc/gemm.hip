@@ -288,7 +288,7 @@ static int gemm_impl() {
 // many half-empty tiles and frequent changes of the b operand).  Crossovers measured on MI355X
 // inside a training step (operands freshly written, i.e. partly cache-resident):
 //   dense      pipelined from K = 512 on (+5 % at 512, +13..20 % from 2048 on)
-//   m-grouped  pipelined for >= 1536 rows per group and K >= 2048 (+3..13 %); below, -2..-9 %
+//   m-grouped  pipelined for >= 1536 rows per group and K >= 2048 (+3..13 %); below, -1..-9 %
 //   k-grouped  pipelined for >= 6 blocks of 128 rows per group (+0..6 %); at 4.5 blocks, -5..-9 %
 static bool prefer_pipelined(const GemmArgs& g) {
   switch (g.mode) {

@@ -255,7 +255,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
     // ---- epilogue ----
     if (!wave_active) continue;
     if (MODE == GEMM_K_GROUPED && nk == 0 && ACC) continue;
-    store_tile<MODE, TM, TN, ACC, false>(acc, p, C, wm0, wn0, lane, lds + NS * STAGE + SC_RING * (BM + BN) * 4 + 512 + wave * 2048);
+    store_tile<MODE, TM, TN, ACC, 0>(acc, p, C, wm0, wn0, lane, lds + NS * STAGE + SC_RING * (BM + BN) * 4 + 512 + wave * 2048);
   }
   wait_all_vmem();  // nothing may still be writing into this workgroup's LDS when it retires
 }

@@ -168,15 +168,17 @@ struct Tile {
 // 2 * op_sel_hi bit, one pair per operand).  Issued as volatile inline assembly with a memory
 // clobber: the compiler keeps such statements, and every memory operation between them, in source
 // order, which is what pins the interleaving of MFMAs, LDS reads and direct-to-LDS loads in the
-// main loop.  The accumulator lives in the accumulation registers ("a" constraint).
+// main loop.  AGPR: the accumulator lives in the accumulation registers ("a" constraint), which a
+// wave with 256 accumulator values needs; with 128 it lives in ordinary registers ("v"), where the
+// epilogue reads it without a copy and shares one register pool with everything else.
+template <bool AGPR>
 __device__ __forceinline__ void mfma_sel(const v8i& a, const v8i& b, v16f& c, int ia, int sa, int ib, int sb) {
-#define PT_MFMA(IA, IB, S0, S1, H0, H1)                                                                         \
-  case IA * 4 + IB:                                                                                             \
-    asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[" #S0 "," #S1 ",0] op_sel_hi:[" #H0 \
-                 "," #H1 ",0]"                                                                                  \
-                 : "+a"(c)                                                                                      \
-                 : "v"(a), "v"(b), "v"(sa), "v"(sb)                                                             \
-                 : "memory");                                                                                   \
+#define PT_MFMA_TEXT(S0, S1, H0, H1) \
+  "v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[" #S0 "," #S1 ",0] op_sel_hi:[" #H0 "," #H1 ",0]"
+#define PT_MFMA(IA, IB, S0, S1, H0, H1)                                                                                  \
+  case IA * 4 + IB:                                                                                                      \
+    if constexpr (AGPR) asm volatile(PT_MFMA_TEXT(S0, S1, H0, H1) : "+a"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb) : "memory"); \
+    else asm volatile(PT_MFMA_TEXT(S0, S1, H0, H1) : "+v"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb) : "memory");               \
     break;
   switch (ia * 4 + ib) {
     PT_MFMA(0, 0, 0, 0, 0, 0) PT_MFMA(0, 1, 0, 1, 0, 0) PT_MFMA(0, 2, 0, 0, 0, 1) PT_MFMA(0, 3, 0, 1, 0, 1)
@@ -185,6 +187,7 @@ __device__ __forceinline__ void mfma_sel(const v8i& a, const v8i& b, v16f& c, in
     PT_MFMA(3, 0, 1, 0, 1, 0) PT_MFMA(3, 1, 1, 1, 1, 0) PT_MFMA(3, 2, 1, 0, 1, 1) PT_MFMA(3, 3, 1, 1, 1, 1)
   }
 #undef PT_MFMA
+#undef PT_MFMA_TEXT
 }
 
 // s_pref[g] = number of BM-row tiles of groups < g (s_pref[G] = their total), from the cumulative
@@ -267,11 +270,19 @@ __device__ __forceinline__ void decode_tile(const GemmArgs& p, const int* s_pref
   }
 }
 
+// Hands one accumulator block produced by inline-assembly MFMAs to the compiler: PIN 1 = it lives
+// in the accumulation registers, 2 = in ordinary registers, 0 = the compiler produced it itself.
+template <int PIN>
+__device__ __forceinline__ void pin_acc(v16f& a) {
+  if constexpr (PIN == 1) asm volatile("" : "+a"(a));
+  else if constexpr (PIN == 2) asm volatile("" : "+v"(a));
+}
+
 // Writes one wave's TM x TN blocks of 32 x 32 results of tile T (rows wm0.., columns wn0.. of the
-// tile).  `stg` is the wave's 2 KiB LDS staging area.  PIN: the accumulators were produced by
-// inline-assembly MFMAs and live in the accumulation registers; each block is handed to the
-// compiler only right before its store, so that it is copied out one block at a time.
-template <int MODE, int TM, int TN, bool ACC, bool PIN>
+// tile).  `stg` is the wave's 2 KiB LDS staging area.  PIN != 0: the accumulators were produced by
+// inline-assembly MFMAs; each block is handed to the compiler only right before its store, so
+// that it is converted and copied out one block at a time.
+template <int MODE, int TM, int TN, bool ACC, int PIN>
 __device__ __forceinline__ void store_tile(v16f (&acc)[TM][TN], const GemmArgs& p, const Tile& T, int wm0, int wn0, int lane,
                                            uint8_t* stg) {
   const uint32_t esz = p.out_dtype == PT_F32 ? 4 : 2;
@@ -306,7 +317,7 @@ __device__ __forceinline__ void store_tile(v16f (&acc)[TM][TN], const GemmArgs& 
         uint32_t voff[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) voff[q] = colc < T.b_lim ? vrow[q] : kOob;
-        if constexpr (PIN) { asm volatile("" : "+a"(acc[i][j])); asm volatile("" : "+a"(acc[i][j + 1])); }
+        pin_acc<PIN>(acc[i][j]); pin_acc<PIN>(acc[i][j + 1]);
         store_staged_bf16_lines(acc[i][j], acc[i][j + 1], rs_sc, stg, voff, (uint32_t)(T.b_row0 + wn0 + j * 32) * 2, false, lane);
       }
     }
@@ -323,7 +334,7 @@ __device__ __forceinline__ void store_tile(v16f (&acc)[TM][TN], const GemmArgs& 
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           voff[q] = colc < T.b_lim ? (uint32_t)(q * 8 + (lane >> 3)) * pitch + (uint32_t)(lane & 7) * 16 : kOob;
-        if constexpr (PIN) { asm volatile("" : "+a"(acc[i][j])); asm volatile("" : "+a"(acc[i][j + 1])); }
+        pin_acc<PIN>(acc[i][j]); pin_acc<PIN>(acc[i][j + 1]);
         store_staged_bf16_lines(acc[i][j], acc[i][j + 1], rs_out, stg, voff, s_tile + i * 32 * pitch + j * 64, ACC, lane, has_bias, bias);
       }
     }
@@ -333,21 +344,21 @@ __device__ __forceinline__ void store_tile(v16f (&acc)[TM][TN], const GemmArgs& 
     for (int j = 0; j < TN; ++j) {
       const uint32_t voff = colw + j * 32 < T.b_lim ? (uint32_t)(4 * (lane >> 5) + odd) * pitch + (uint32_t)(((lane & 31) & ~1) + j * 32) * 2 : kOob;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) { if constexpr (PIN) asm volatile("" : "+a"(acc[i][j])); store_pairs_bf16(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC, odd); }
+      for (int i = 0; i < TM; ++i) { pin_acc<PIN>(acc[i][j]); store_pairs_bf16(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC, odd); }
     }
   } else if (p.out_dtype == PT_F32) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const uint32_t voff = colw + j * 32 < T.b_lim ? (uint32_t)(4 * (lane >> 5)) * pitch + (uint32_t)((lane & 31) + j * 32) * 4 : kOob;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) { if constexpr (PIN) asm volatile("" : "+a"(acc[i][j])); store_f32(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC); }
+      for (int i = 0; i < TM; ++i) { pin_acc<PIN>(acc[i][j]); store_f32(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC); }
     }
   } else {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const uint32_t voff = colw + j * 32 < T.b_lim ? (uint32_t)(4 * (lane >> 5)) * pitch + (uint32_t)((lane & 31) + j * 32) * 2 : kOob;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) { if constexpr (PIN) asm volatile("" : "+a"(acc[i][j])); store_single_bf16(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC); }
+      for (int i = 0; i < TM; ++i) { pin_acc<PIN>(acc[i][j]); store_single_bf16(acc[i][j], rs_out, voff, s_tile + i * 32 * pitch, pitch, ACC); }
     }
   }
 }

@@ -9,8 +9,9 @@
 //    the address arithmetic and the M0 writes hide under the matrix pipe as well;
 //  * one workgroup barrier per 128-block instead of two;
 //  * the MFMAs are volatile inline assembly with a memory clobber, which pins this interleaving
-//    (the compiler's scheduler would otherwise regroup reads and MFMAs), and keeps the
-//    accumulators in the accumulation registers for the whole tile;
+//    (the compiler's scheduler would otherwise regroup reads and MFMAs); the accumulators of the
+//    8-wave shape stay in ordinary registers, where the epilogue reads them without a copy, those
+//    of the 4-wave shape (256 values per lane) in the accumulation registers;
 //  * the E8M0 exponent bytes of a block's scales are packed four to a register and selected by
 //    the MFMA's op_sel bits.
 //
@@ -31,6 +32,9 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_pipelined_kerne
   constexpr int NW = WGM * WGN;
   constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int TM = WM / 32, TN = WN / 32;
+  // 128 accumulator values per lane fit next to everything else in the 256 ordinary registers a
+  // wave has at two waves per SIMD; 256 need the accumulation registers.
+  constexpr bool kAccInAgpr = TM * TN * 16 > 128;
   constexpr int BK = 128;                      // reduction depth of one stage = one scale block = two MFMA steps
   constexpr int NS = 2;                        // stages in the LDS ring
   constexpr int STAGE = (BM + BN) * BK;
@@ -290,7 +294,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_pipelined_kerne
       auto half_a = [&](auto act) {
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
-          mfma_sel(fa0[m / TN], fb0[m % TN], acc[m / TN][m % TN], m / TN, sca, m % TN, scb);
+          mfma_sel<kAccInAgpr>(fa0[m / TN], fb0[m % TN], acc[m / TN][m % TN], m / TN, sca, m % TN, scb);
 #pragma unroll
           for (int r = m * NR / NM; r < (m + 1) * NR / NM; ++r) read_frag_piece(gb, 1, r, fa1, fb1);
           __builtin_amdgcn_sched_barrier(0);
@@ -299,7 +303,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_pipelined_kerne
       auto half_b = [&](auto act) {
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
-          mfma_sel(fa1[m / TN], fb1[m % TN], acc[m / TN][m % TN], m / TN, sca, m % TN, scb);
+          mfma_sel<kAccInAgpr>(fa1[m / TN], fb1[m % TN], acc[m / TN][m % TN], m / TN, sca, m % TN, scb);
           // the direct-to-LDS loads go out in the first DMA_SLOTS MFMA slots: the earlier they start,
           // the longer they have before the next stage's barrier
           if (m < DMA_SLOTS) {
@@ -328,7 +332,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_pipelined_kerne
     // ---- epilogue ----
     if (!wave_active) continue;
     if (MODE == GEMM_K_GROUPED && nk == 0 && ACC) continue;
-    store_tile<MODE, TM, TN, ACC, true>(acc, p, C, wm0, wn0, lane, lds + NS * STAGE + SC_RING * (BM + BN) * 4 + 512 + wave * 2048);
+    store_tile<MODE, TM, TN, ACC, kAccInAgpr ? 1 : 2>(acc, p, C, wm0, wn0, lane, lds + NS * STAGE + SC_RING * (BM + BN) * 4 + 512 + wave * 2048);
   }
   wait_all_vmem();  // nothing may still be writing into this workgroup's LDS when it retires
 }

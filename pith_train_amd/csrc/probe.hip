@@ -13,8 +13,9 @@ __global__ __launch_bounds__(256) void mfma_rate_probe_kernel(float* sink, int i
   probe_v8i a, b;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    a[i] = (int)threadIdx.x * 3 + i;
-    b[i] = (int)threadIdx.x * 7 + i;
+    // e4m3 bytes 0x30..0x3F (0.5 .. 1.875), varying by lane and register: finite sums, live operand bits
+    a[i] = 0x30303030 + (((int)threadIdx.x * 0x01030507 + i * 0x02040608) & 0x0F0F0F0F);
+    b[i] = 0x30303030 + (((int)threadIdx.x * 0x07050301 + i * 0x08060402) & 0x0F0F0F0F);
   }
   probe_v16f acc[8];
 #pragma unroll
