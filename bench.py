@@ -261,7 +261,11 @@ def hbm_kernel_report(H, I, E, rows, eidx, top_k=8, kind="fused", extras=None):
     o = silu_mul_halves(gur)
     rep("silu_mul_2d_kernel bwd [Mp,I]", timeit(lambda: torch.autograd.grad(o, gur, dh, retain_graph=True)), Mp * I * 10)
     del gu, dh, gur, o
-    rep("group_rows + permute_rows_kernel (scatter_for_grouped_gemm) [rows,H]",
+    pbuf = torch.empty((src_of.shape[0], H), device="cuda", dtype=torch.bfloat16)
+    rep("permute_rows_kernel alone (row copy of the scatter, indices given) [rows,H]",
+        timeit(lambda: TS.permute_rows(src, src_of, pbuf, offs[E - 1:])), (rows + Mp) * H * 2 + 4 * src_of.shape[0])
+    del pbuf
+    rep("group_rows + permute_rows_kernel + host copy of the group sizes (scatter_for_grouped_gemm) [rows,H]",
         timeit(lambda: TS.scatter_for_grouped_gemm(src, eidx, E)), (rows + Mp) * H * 2 + 16 * rows)
     rep("gather_rows_kernel (padded_index_gather) [rows,H]", timeit(lambda: TS.padded_index_gather(xp, reverse)),
         2 * rows * H * 2 + 8 * rows)
