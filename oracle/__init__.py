@@ -26,4 +26,12 @@ formulations (see ``tests/test_oracle_*.py``):
   force, and the invariants the reference's own tests assert.
 * epilogues                  - closed forms vs ``torch.autograd`` of the
   textbook expression.
+* combine (both branches)    - bit for bit against the reference's tensor
+  expression where the sum has one order, a scalar loop in row order, known
+  answers that separate the rounding rules, autograd for the backward.
+* router gate                - ``torch.topk`` where no values tie, closed
+  forms, a scalar loop over ``math.exp``, a hand-worked group limit.
+* cross-entropy              - ``F.cross_entropy`` in float64 (loss, per-row
+  loss, autograd gradient), the closed form for uniform logits, the
+  two-rounding rule at the target, the ignore rules.
 """
