@@ -16,6 +16,7 @@ import torch
 from .. import _lib
 from .deepgemm_quantize import FP8, fp8cast_rowwise_colwise_t, fp8cast_rowwise_colwise_t_rows
 from .grouped_linear import m_grouped_fp8_gemm_nt, schedule_wgrad
+from .token_scatter import _GEMM_ALLOC_ALIGNMENT, _PaddedIndexGather
 
 
 def _cdiv(a: int, b: int) -> int:
@@ -143,9 +144,7 @@ def _backward(ctx, grad_out):
     if expand_idx is not None:
         # one gradient row per routed row so far: rows that expand the same source row are summed
         # (the backward of the expanding gather, token_scatter.py:311-325)
-        from .token_scatter import _PaddedIndexGather
-
-        grad_x = _PaddedIndexGather.scatter_sum(grad_x, expand_idx, rows_src, 1024)
+        grad_x = _PaddedIndexGather.scatter_sum(grad_x, expand_idx, rows_src, _GEMM_ALLOC_ALIGNMENT)
     if isinstance(ctx.gate_up_weights, tuple):
         # separate gate and up parameters: each gets the weight-gradient GEMM of its half of the
         # colwise twin (rows of the transposed bytes, columns of the scale array)
