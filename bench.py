@@ -132,7 +132,8 @@ def build_module(kind, H, I, E, w):
 class GemmTimer:
     """HIP events (on the stream the kernels are launched on) around every GEMM entry point."""
 
-    NAMES = ("pt_gemm_m_grouped_nt", "pt_gemm_m_grouped_nt_scatter", "pt_gemm_m_grouped_nt_bias", "pt_gemm_k_grouped_wgrad",
+    NAMES = ("pt_gemm_m_grouped_nt", "pt_gemm_m_grouped_nt_scatter", "pt_gemm_m_grouped_nt_bias",
+             "pt_gemm_m_grouped_nt_scatter_bias", "pt_gemm_k_grouped_wgrad",
              "pt_gemm_k_grouped_wgrad_ld",
              "pt_gemm_nt_dense")
 

@@ -153,6 +153,14 @@ int pt_gemm_m_grouped_nt_bias(const void* a_fp8, const float* a_scale, const voi
                               const float* b_scale, void* out, int out_dtype, const int32_t* offs,
                               int32_t num_groups, int64_t M, int64_t N, int64_t K,
                               const void* bias, pt_stream_t stream);
+/* Both of the above: the bias row of the group is added to the rounded result and the row is
+ * stored at out[out_row_index[r]] (grouped linear + indexed_bias_add + the un-permuting
+ * padded_index_gather of forward_stage3, models/gpt_oss.py:155-156,318-321, as one kernel). */
+int pt_gemm_m_grouped_nt_scatter_bias(const void* a_fp8, const float* a_scale, const void* b_fp8,
+                                      const float* b_scale, void* out, int out_dtype,
+                                      const int32_t* offs, int32_t num_groups, int64_t M, int64_t N,
+                                      int64_t K, const int32_t* out_row_index, int64_t out_rows,
+                                      const void* bias, pt_stream_t stream);
 
 /* dW[g][n,k] = sum_{m in group g} dY[m,n] X[m,k] with colwise-quantised operands stored
  * transposed: dy_t[N,M] and x_t[K,M] (PT_CH_TRANSPOSED) and their scales dy_scale[M/128,N],
@@ -307,6 +315,12 @@ int pt_indexed_bias_add_fwd(const void* x, const void* bias, const int64_t* grou
  * _segment_sum_kernel, indexed_bias_add.py:20-96 */
 int pt_segment_sum(const void* x, const int32_t* offs, int32_t num_groups, void* out, int64_t M,
                    int64_t H, int dtype, int out_dtype, pt_stream_t stream);
+/* The same sums with grouped row r read from x[row_index[r]] (x [x_rows,H] un-permuted; a negative
+ * index is a padding row): the bias gradient of a grouped linear whose output rows were stored
+ * through row_index, in the grouped order of the rows (same bits as gathering first). */
+int pt_segment_sum_rows(const void* x, int64_t x_rows, const int32_t* row_index, const int32_t* offs,
+                        int32_t num_groups, void* out, int64_t M, int64_t H, int dtype,
+                        int out_dtype, pt_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Top-k weighted combine with the residual: the memory-bound step that follows the expert path.

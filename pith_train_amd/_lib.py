@@ -38,6 +38,7 @@ SIGNATURES = {
     "pt_gemm_nt_dense": (c_int, [P, P, P, P, P, c_int, I64, I64, I64, P]),
     "pt_gemm_m_grouped_nt": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P]),
     "pt_gemm_m_grouped_nt_bias": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, P]),
+    "pt_gemm_m_grouped_nt_scatter_bias": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, I64, P, P]),
     "pt_gemm_m_grouped_nt_scatter": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, I64, P]),
     "pt_gemm_k_grouped_wgrad": (c_int, [P, P, P, P, P, c_int, c_int, P, I32, I64, I64, I64, P]),
     "pt_gemm_k_grouped_wgrad_ld": (c_int, [P, P, I64, P, P, I64, P, c_int, c_int, P, I32, I64, I64, I64, P]),
@@ -72,6 +73,7 @@ SIGNATURES = {
     "pt_clamped_swiglu_bwd": (c_int, [P, P, P, I64, F, F, c_int, P]),
     "pt_indexed_bias_add_fwd": (c_int, [P, P, P, P, I64, I64, c_int, P]),
     "pt_segment_sum": (c_int, [P, P, I32, P, I64, I64, c_int, c_int, P]),
+    "pt_segment_sum_rows": (c_int, [P, I64, P, P, I32, P, I64, I64, c_int, c_int, P]),
 }
 
 _lib = None

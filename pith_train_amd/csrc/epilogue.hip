@@ -208,9 +208,11 @@ __global__ __launch_bounds__(256) void bias_add_kernel(const char* x, const char
 
 // ---- per-group row sums -----------------------------------------------------------------------------
 // grid (ceil(H/128), G); 16 column chunks x 16 row lanes; fp32 accumulate, fixed order.
+// row_index (optional): grouped row r is x[row_index[r]] (negative: a padding row, nothing to add),
+// i.e. the sum runs over the grouped order while x stays un-permuted.
 template <typename S, typename O>
 __global__ __launch_bounds__(256) void segment_sum_kernel(const char* x, const int32_t* offs, char* out, int64_t M,
-                                                          int64_t H, int vec) {
+                                                          int64_t H, int vec, const int32_t* row_index, int64_t x_rows) {
   __shared__ float s[16][129];
   const int g = blockIdx.y;
   const int cc = threadIdx.x & 15, rl = threadIdx.x >> 4;
@@ -223,16 +225,21 @@ __global__ __launch_bounds__(256) void segment_sum_kernel(const char* x, const i
   if (vec) {
     if (h0 < H)
       for (int64_t r = start + rl; r < end; r += 16) {
+        const int64_t src = row_index ? (int64_t)row_index[r] : r;
+        if (src < 0 || src >= x_rows) continue;
         float v[8];
-        S::load8(x + (r * H + h0) * S::kBytes, v);
+        S::load8(x + (src * H + h0) * S::kBytes, v);
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[j] += v[j];
       }
   } else {
-    for (int64_t r = start + rl; r < end; r += 16)
+    for (int64_t r = start + rl; r < end; r += 16) {
+      const int64_t src = row_index ? (int64_t)row_index[r] : r;
+      if (src < 0 || src >= x_rows) continue;
 #pragma unroll
       for (int j = 0; j < 8; ++j)
-        if (h0 + j < H) acc[j] += S::load1(x + (r * H + h0 + j) * S::kBytes);
+        if (h0 + j < H) acc[j] += S::load1(x + (src * H + h0 + j) * S::kBytes);
+    }
   }
 #pragma unroll
   for (int j = 0; j < 8; ++j) s[rl][cc * 8 + j] = acc[j];
@@ -376,14 +383,14 @@ extern "C" int pt_indexed_bias_add_fwd(const void* x, const void* bias, const in
   return check_launch("indexed_bias_add_fwd");
 }
 
-extern "C" int pt_segment_sum(const void* x, const int32_t* offs, int32_t num_groups, void* out, int64_t M, int64_t H,
-                              int dtype, int out_dtype, pt_stream_t stream) {
+static int segment_sum_impl(const void* x, int64_t x_rows, const int32_t* row_index, const int32_t* offs, int32_t num_groups,
+                            void* out, int64_t M, int64_t H, int dtype, int out_dtype, pt_stream_t stream) {
   if (num_groups == 0 || H == 0) return PT_OK;
-  PT_REQUIRE(num_groups > 0 && num_groups <= 65535 && H > 0 && M >= 0 && x && offs && out, "segment_sum: bad arguments");
+  PT_REQUIRE(num_groups > 0 && num_groups <= 65535 && H > 0 && M >= 0 && x_rows >= 0 && x && offs && out, "segment_sum: bad arguments");
   const int vec = (H % 8 == 0) && aligned16(x);
   dim3 grid((unsigned)cdiv(H, 128), (unsigned)num_groups);
   hipStream_t s = (hipStream_t)stream;
-#define PT_SEG(SI, SO) segment_sum_kernel<SI, SO><<<grid, 256, 0, s>>>((const char*)x, offs, (char*)out, M, H, vec)
+#define PT_SEG(SI, SO) segment_sum_kernel<SI, SO><<<grid, 256, 0, s>>>((const char*)x, offs, (char*)out, M, H, vec, row_index, x_rows)
   if (dtype == PT_BF16 && out_dtype == PT_BF16) PT_SEG(st_bf16, st_bf16);
   else if (dtype == PT_BF16 && out_dtype == PT_F32) PT_SEG(st_bf16, st_f32);
   else if (dtype == PT_F16 && out_dtype == PT_F16) PT_SEG(st_f16, st_f16);
@@ -393,4 +400,16 @@ extern "C" int pt_segment_sum(const void* x, const int32_t* offs, int32_t num_gr
   else PT_REQUIRE(false, "segment_sum: unsupported dtype pair %d -> %d", dtype, out_dtype);
 #undef PT_SEG
   return check_launch("segment_sum");
+}
+
+extern "C" int pt_segment_sum(const void* x, const int32_t* offs, int32_t num_groups, void* out, int64_t M, int64_t H,
+                              int dtype, int out_dtype, pt_stream_t stream) {
+  return segment_sum_impl(x, M, nullptr, offs, num_groups, out, M, H, dtype, out_dtype, stream);
+}
+
+extern "C" int pt_segment_sum_rows(const void* x, int64_t x_rows, const int32_t* row_index, const int32_t* offs,
+                                   int32_t num_groups, void* out, int64_t M, int64_t H, int dtype, int out_dtype,
+                                   pt_stream_t stream) {
+  PT_REQUIRE(row_index, "segment_sum_rows: null row_index");
+  return segment_sum_impl(x, x_rows, row_index, offs, num_groups, out, M, H, dtype, out_dtype, stream);
 }

@@ -372,8 +372,8 @@ static int gemm_m_grouped_impl(const void* a_fp8, const float* a_scale, const vo
     g.out_row_index = out_row_index; g.out_rows = out_rows;
   }
   if (bias) {
-    PT_REQUIRE(!out_row_index && N % 8 == 0 && al16(out) && al16(bias),
-               "gemm_m_grouped_nt_bias: needs N %% 8 == 0 and 16-byte aligned output and bias, and no scattered rows");
+    PT_REQUIRE(N % 8 == 0 && al16(out) && al16(bias),
+               "gemm_m_grouped_nt_bias: needs N %% 8 == 0 and 16-byte aligned output and bias");
     g.bias = bias;
   }
   return dispatch_gemm(g, (hipStream_t)stream);
@@ -390,6 +390,15 @@ extern "C" int pt_gemm_m_grouped_nt_scatter(const void* a_fp8, const float* a_sc
                                             int64_t K, const int32_t* out_row_index, int64_t out_rows, pt_stream_t stream) {
   PT_REQUIRE(out_row_index, "gemm_m_grouped_nt_scatter: null out_row_index");
   return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, out_row_index, out_rows, nullptr,
+                             stream);
+}
+
+extern "C" int pt_gemm_m_grouped_nt_scatter_bias(const void* a_fp8, const float* a_scale, const void* b_fp8,
+                                                 const float* b_scale, void* out, int out_dtype, const int32_t* offs, int32_t G,
+                                                 int64_t M, int64_t N, int64_t K, const int32_t* out_row_index, int64_t out_rows,
+                                                 const void* bias, pt_stream_t stream) {
+  PT_REQUIRE(out_row_index && bias, "gemm_m_grouped_nt_scatter_bias: null out_row_index or bias");
+  return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, out_row_index, out_rows, bias,
                              stream);
 }
 

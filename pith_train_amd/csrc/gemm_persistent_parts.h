@@ -317,8 +317,11 @@ __device__ __forceinline__ void store_tile(v16f (&acc)[TM][TN], const GemmArgs& 
         uint32_t voff[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) voff[q] = colc < T.b_lim ? vrow[q] : kOob;
+        v4i bias = v4i{0, 0, 0, 0};
+        if (p.bias != nullptr && colc < T.b_lim) bias = *(const v4i*)((const char*)p.bias + ((int64_t)T.g * p.rows_b + colc) * 2);
         pin_acc<PIN>(acc[i][j]); pin_acc<PIN>(acc[i][j + 1]);
-        store_staged_bf16_lines(acc[i][j], acc[i][j + 1], rs_sc, stg, voff, (uint32_t)(T.b_row0 + wn0 + j * 32) * 2, false, lane);
+        store_staged_bf16_lines(acc[i][j], acc[i][j + 1], rs_sc, stg, voff, (uint32_t)(T.b_row0 + wn0 + j * 32) * 2, false, lane,
+                                p.bias != nullptr, bias);
       }
     }
   } else if (p.out_dtype != PT_F32 && wide_ok && (T.b_lim & 7) == 0) {

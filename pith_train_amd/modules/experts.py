@@ -147,6 +147,9 @@ class GptOssExperts(nn.Module):
         self.down_proj_bias = nn.Parameter(torch.zeros(num_experts, hidden_size))
         self._wq_cache: dict | None = None
         self._wq_version: int = -1
+        # extension: the two indexed_bias_add steps happen in the stores of the GEMMs before them
+        # (same bits) wherever the shapes and dtypes allow it
+        self.fuse_bias = True
 
     def _quantized_weight(self, name: str, weight: torch.Tensor):
         if torch.compiler.is_compiling():
@@ -160,33 +163,42 @@ class GptOssExperts(nn.Module):
             cache[name] = fp8cast_blockwise_transpose_batched(weight)
         return cache[name]
 
-    def _group_linear(self, x, weight, name, offs, ks, ks_tensor, group_indices_, in_rows=None, bias=None):
+    def _group_linear(self, x, weight, name, offs, ks, ks_tensor, group_indices_, in_rows=None, bias=None,
+                      out_rows=None, out_m=None):
         if x.shape[0] == 0:
             return x @ weight[0].transpose(-2, -1)
         if training.fp8:
             return FP8GroupedLinearFunc.apply(
                 x, weight, offs, ks, ks_tensor, self._quantized_weight(name, weight), group_indices_, in_rows,
-                None, None, bias,
+                out_rows, out_m, bias,
             )
         assert in_rows is None, "row maps need the FP8 layers"
         return GroupedLinearFunc.apply(x, weight, offs)
 
-    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None, fuse_bias: bool = True):
+    def bias_fusable(self, x) -> bool:
+        """Whether the two ``indexed_bias_add`` steps happen in the stores of the GEMMs."""
+        return (self.fuse_bias and training.fp8 and x.shape[0] > 0 and x.dtype == torch.bfloat16
+                and self.gate_up_proj_bias.dtype == x.dtype and self.down_proj_bias.dtype == x.dtype
+                and self.gate_up_proj.shape[1] % 8 == 0 and self.down_proj.shape[1] % 8 == 0)
+
+    def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None, scatter_output: bool = False):
         """``row_map`` (extension, FP8 only): the scatter's int32 source-row map; ``x`` is then the
-        un-permuted token tensor and the first quantisation gathers its rows (the result stays in
-        the grouped layout: the per-group bias gradients are sums over contiguous row ranges).
-        ``fuse_bias`` (FP8 only): the two ``indexed_bias_add`` steps happen in the stores of the
-        GEMMs before them (same bits)."""
+        un-permuted token tensor and the first quantisation gathers its rows.  The result stays
+        in the grouped layout unless ``scatter_output`` is set (with ``row_map`` and the fused
+        biases): then the last GEMM stores every row, bias added, at its un-permuted place, and
+        the backward sums the bias gradient over the grouped order through the same map.
+        With ``self.fuse_bias`` (FP8 only) the two ``indexed_bias_add`` steps happen in the stores
+        of the GEMMs before them (same bits)."""
         M = x.shape[0] if row_map is None else row_map.shape[0]
-        fused = (fuse_bias and training.fp8 and x.shape[0] > 0 and x.dtype == torch.bfloat16
-                 and self.gate_up_proj_bias.dtype == x.dtype and self.down_proj_bias.dtype == x.dtype
-                 and self.gate_up_proj.shape[1] % 8 == 0 and self.down_proj.shape[1] % 8 == 0)
+        fused = self.bias_fusable(x)
+        assert not scatter_output or (fused and row_map is not None), "scatter_output needs row_map and the fused biases"
         if fused:
             gate_up = self._group_linear(x, self.gate_up_proj, "gate_up_proj", grouped_mm_offs, ks, ks_tensor, None, row_map,
                                          self.gate_up_proj_bias)
             activated = clamped_swiglu(gate_up, 1.702, self.swiglu_limit)
             return self._group_linear(activated, self.down_proj, "down_proj", grouped_mm_offs, ks, ks_tensor, None, None,
-                                      self.down_proj_bias)
+                                      self.down_proj_bias, row_map if scatter_output else None,
+                                      x.shape[0] if scatter_output else None)
         group_ids = group_indices(grouped_mm_offs, M, torch.int64)
         gate_up = self._group_linear(x, self.gate_up_proj, "gate_up_proj", grouped_mm_offs, ks, ks_tensor, None, row_map)
         gate_up = indexed_bias_add(gate_up, self.gate_up_proj_bias, group_ids, grouped_mm_offs)
@@ -234,9 +246,13 @@ def forward_stage3(experts: nn.Module, gathered_tokens, expert_idxs, experts_per
                            expand_idx=expand_idx)
     if (fuse_permute and expand_idx is None and training.fp8 and expert_idxs.shape[0] > 0
             and isinstance(experts, GptOssExperts)):
-        # input side only: the output keeps the grouped layout for the per-group bias sums
         reverse_shuffle_idxs, grouped_mm_offs, ks, ks_tensor, src_of = group_rows_with_sizes(
             expert_idxs, experts_per_rank, device=gathered_tokens.device)
+        if experts.bias_fusable(gathered_tokens):
+            # both sides: rows gathered by the first quantisation, stored un-permuted (bias added)
+            # by the last GEMM; the bias gradients are summed through the same map
+            return experts(gathered_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, row_map=src_of, scatter_output=True)
+        # input side only: the unfused bias add wants the grouped layout
         outs = experts(gathered_tokens, grouped_mm_offs, ks=ks, ks_tensor=ks_tensor, row_map=src_of)
         return padded_index_gather(outs, reverse_shuffle_idxs)
     pre = None

@@ -111,12 +111,22 @@ def m_grouped_fp8_gemm_nt(a, b, out: torch.Tensor, grouped_mm_offs: torch.Tensor
     scale[G,N/128,K/128]).  Rows at or past ``grouped_mm_offs[-1]`` are left untouched.  With
     ``out_rows`` (int32 [M]) result row r is written to ``out[out_rows[r]]`` instead (negative:
     dropped).  With ``bias`` ([G, N] in ``out``'s dtype) the bias row of a row's group is added
-    to the rounded result (``out + bias[group_ids]`` in the output dtype, as one kernel)."""
+    to the rounded result (``out + bias[group_ids]`` in the output dtype, as one kernel).  Both
+    may be given."""
     (a_fp8, a_s), (b_fp8, b_s) = a, b
     M, K = a_fp8.shape
     G, N, _ = b_fp8.shape
     if bias is not None:
-        assert out_rows is None and bias.shape == (G, N) and bias.dtype == out.dtype and bias.is_contiguous()
+        assert bias.shape == (G, N) and bias.dtype == out.dtype and bias.is_contiguous()
+    if bias is not None and out_rows is not None:
+        assert out_rows.dtype == torch.int32 and out_rows.shape == (M,)
+        _lib.call(
+            "pt_gemm_m_grouped_nt_scatter_bias", a_fp8.data_ptr(), a_s.data_ptr(), b_fp8.data_ptr(), b_s.data_ptr(),
+            out.data_ptr(), _lib.dtype_code(out.dtype), grouped_mm_offs.data_ptr(), G, M, N, K,
+            out_rows.contiguous().data_ptr(), out.shape[0], bias.data_ptr(), _lib.stream_ptr(out.device),
+        )  # fmt: skip
+        return out
+    if bias is not None:
         _lib.call(
             "pt_gemm_m_grouped_nt_bias", a_fp8.data_ptr(), a_s.data_ptr(), b_fp8.data_ptr(), b_s.data_ptr(),
             out.data_ptr(), _lib.dtype_code(out.dtype), grouped_mm_offs.data_ptr(), G, M, N, K, bias.data_ptr(),
@@ -277,7 +287,8 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
         if ctx.bias_dtype is not None:
             from .indexed_bias_add import _segment_sum_along_rows
 
-            grad_bias = _segment_sum_along_rows(grad_output, offs, ctx.bias_dtype)
+            # un-permuted gradient: summed in the grouped order of its rows through the row map
+            grad_bias = _segment_sum_along_rows(grad_output, offs, ctx.bias_dtype, out_rows)
         return grad_input, None, None, None, None, None, None, None, None, None, grad_bias
 
 

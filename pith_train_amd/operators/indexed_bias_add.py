@@ -12,10 +12,14 @@ import torch
 from .. import _lib
 
 
-def _segment_sum_along_rows(x: torch.Tensor, grouped_mm_offs: torch.Tensor, out_dtype: torch.dtype):
-    """(E, H) per-group row sums, fp32 accumulation in a fixed order, stored as ``out_dtype``."""
+def _segment_sum_along_rows(x: torch.Tensor, grouped_mm_offs: torch.Tensor, out_dtype: torch.dtype,
+                            row_index: torch.Tensor | None = None):
+    """(E, H) per-group row sums, fp32 accumulation in a fixed order, stored as ``out_dtype``.
+    With ``row_index`` (int32 ``[M]``) grouped row r is ``x[row_index[r]]`` (negative: padding),
+    ``x`` being the un-permuted ``[m, H]`` tensor: the same sums, in the same order, as over
+    ``x`` gathered into the grouped layout."""
     assert x.is_contiguous(), "x must be contiguous"
-    M, H = x.shape
+    M, H = (row_index.shape[0], x.shape[1]) if row_index is not None else x.shape
     E = grouped_mm_offs.shape[0]
     offs = grouped_mm_offs.to(torch.int32).contiguous()
     direct = (x.dtype, out_dtype) in {
@@ -25,7 +29,12 @@ def _segment_sum_along_rows(x: torch.Tensor, grouped_mm_offs: torch.Tensor, out_
     }  # fmt: skip
     kdtype = out_dtype if direct else torch.float32
     out = torch.empty((E, H), dtype=kdtype, device=x.device)
-    if E and H:
+    if E and H and row_index is not None:
+        _lib.call(
+            "pt_segment_sum_rows", x.data_ptr(), x.shape[0], row_index.contiguous().data_ptr(), offs.data_ptr(), E,
+            out.data_ptr(), M, H, _lib.dtype_code(x.dtype), _lib.dtype_code(kdtype), _lib.stream_ptr(x.device),
+        )  # fmt: skip
+    elif E and H:
         _lib.call(
             "pt_segment_sum", x.data_ptr(), offs.data_ptr(), E, out.data_ptr(), M, H,
             _lib.dtype_code(x.dtype), _lib.dtype_code(kdtype), _lib.stream_ptr(x.device),

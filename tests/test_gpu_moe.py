@@ -293,10 +293,9 @@ def test_dense_mlp_and_bf16_switch():
 
 @pytest.mark.parametrize("kind,E,H,I,T,k,zipf", [c for c in CASES if c[0] == "gpt_oss"] + [("gpt_oss", 8, 512, 256, 900, 4, 1.2)])
 def test_gpt_oss_bias_folded_into_the_gemm_store_is_bit_identical(kind, E, H, I, T, k, zipf):
-    """indexed_bias_add done by the store of the GEMM before it: same output, same token, weight
-    and bias gradients as the separate operator."""
-    import functools
-
+    """indexed_bias_add done by the store of the GEMM before it, and the un-permuting gather done
+    by the same store: same output, same token, weight and bias gradients as the separate
+    operators."""
     from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
     from pith_train_amd.modules.experts import forward_stage3
 
@@ -306,15 +305,20 @@ def test_gpt_oss_bias_folded_into_the_gemm_store_is_bit_identical(kind, E, H, I,
     dy = torch.randn((T * k, H), generator=g).bfloat16().cuda()
     w = _weights(kind, E, H, I, 8)
     res = []
-    for fuse_bias in (True, False):
+    # (fuse_bias, fuse_permute): the default runs everything inside the GEMMs and the
+    # quantisations - rows gathered by the first quantisation, biases added and rows stored at
+    # their un-permuted place by the GEMMs, bias gradients summed through the row map
+    for fuse_bias, fuse_permute in ((True, True), (False, True), (True, False), (False, False)):
         mod, params = _build(kind, E, H, I, w)
-        mod.forward = functools.partial(mod.forward, fuse_bias=fuse_bias)
+        mod.fuse_bias = fuse_bias
         FP8WeightCacheControl.step()
         tok = tokens.clone().requires_grad_(True)
-        out = forward_stage3(mod, tok, ids.reshape(-1).cuda(), E)
+        out = forward_stage3(mod, tok, ids.reshape(-1).cuda(), E, fuse_permute=fuse_permute)
+        assert out.shape == (T * k, H)
         out.backward(dy)
         res.append((out.detach(), tok.grad, {n: p.grad for n, p in params.items()}))
-    assert torch.equal(res[0][0], res[1][0]), "forward output differs"
-    assert torch.equal(res[0][1], res[1][1]), "token gradient differs"
-    for n in res[0][2]:
-        assert torch.equal(res[0][2][n], res[1][2][n]), f"{n} gradient differs"
+    for other in res[1:]:
+        assert torch.equal(res[0][0], other[0]), "forward output differs"
+        assert torch.equal(res[0][1], other[1]), "token gradient differs"
+        for n in res[0][2]:
+            assert torch.equal(res[0][2][n], other[2][n]), f"{n} gradient differs"
