@@ -35,7 +35,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
                 "every wave must issue the same number of loads per stage");
   constexpr int SC_RING = NS;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [NS][STAGE] operand stages | [SC_RING][BM+BN] fp32 scales
-  __shared__ int s_pref[MODE == GEMM_M_GROUPED ? kMaxGroupsGemm + 1 : 1];
+  __shared__ int s_pref[MODE != GEMM_DENSE ? kMaxGroupsGemm + 1 : 1];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -51,13 +51,14 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
     total_tiles = __builtin_amdgcn_readfirstlane(s_pref[p.G]) * p.tiles_b;
   } else {
     total_tiles = (int)p.total_tiles;
+    if (MODE == GEMM_K_GROUPED) scan_group_costs(p, s_pref, tid, lane);
   }
-  const int per_xcd = (total_tiles + 7) / 8;
   const int xcd = blockIdx.x & 7;
-  int t_end = (xcd + 1) * per_xcd;
-  if (t_end > total_tiles) t_end = total_tiles;
+  // lanes 0 and 1 find the two ends of this XCD's share of the list side by side
+  const int t_cut = xcd_first_tile<MODE>(p, s_pref, total_tiles, xcd + (lane & 1));
+  const int t_end = __builtin_amdgcn_readlane(t_cut, 1);
   const int t_step = gridDim.x >> 3;
-  const int t_first = xcd * per_xcd + (blockIdx.x >> 3);
+  const int t_first = __builtin_amdgcn_readlane(t_cut, 0) + (blockIdx.x >> 3);
 
   auto decode_any = [&](int t, Tile& T) { decode_tile<MODE, BM, BN>(p, s_pref, t, T); };
 
@@ -281,7 +282,7 @@ static int launch_mode(const GemmArgs& a, hipStream_t stream) {
 }
 
 int launch_gemm_persistent(const GemmArgs& a, int variant, hipStream_t stream) {
-  PT_REQUIRE(a.mode != GEMM_M_GROUPED || a.G <= kMaxGroupsGemm, "gemm: at most %d groups", kMaxGroupsGemm);
+  PT_REQUIRE(a.mode == GEMM_DENSE || a.G <= kMaxGroupsGemm, "gemm: at most %d groups", kMaxGroupsGemm);
   switch (variant) {
     case 0: return launch_mode<256, 256, 2, 4>(a, stream);  // 8 waves, 128 x 64 per wave
   }

@@ -190,17 +190,26 @@ __device__ __forceinline__ void mfma_sel(const v8i& a, const v8i& b, v16f& c, in
 #undef PT_MFMA_TEXT
 }
 
-// s_pref[g] = number of BM-row tiles of groups < g (s_pref[G] = their total), from the cumulative
-// group ends in p.offs; computed by the first wave, followed by a workgroup barrier.
-template <int BM>
-__device__ __forceinline__ void scan_group_tiles(const GemmArgs& p, int* s_pref, int tid, int lane) {
+// s_pref[g] = sum of weight(g') over groups g' < g (s_pref[G] = the total); computed by the first
+// wave, followed by a workgroup barrier.
+template <class W>
+__device__ __forceinline__ void scan_groups(const GemmArgs& p, int* s_pref, int tid, int lane, W weight) {
   if (tid < 64) {
+    // Lane l owns groups [l * per, (l + 1) * per): one global read per group, running sums kept in
+    // LDS, then the lanes' totals are scanned and added to each lane's own entries.
     const int per = (p.G + 63) / 64;
     const int g0 = tid * per;
+    int prev = (g0 > 0 && g0 <= p.G) ? p.offs[g0 - 1] : 0;
     int sum = 0;
+#pragma unroll 4
     for (int q = 0; q < per; ++q) {
       const int g = g0 + q;
-      if (g < p.G) sum += (p.offs[g] - (g ? p.offs[g - 1] : 0) + BM - 1) / BM;
+      if (g < p.G) {
+        const int cur = p.offs[g];
+        sum += weight(cur - prev);
+        prev = cur;
+        s_pref[g + 1] = sum;
+      }
     }
     int incl = sum;
 #pragma unroll
@@ -208,17 +217,55 @@ __device__ __forceinline__ void scan_group_tiles(const GemmArgs& p, int* s_pref,
       const int y = __shfl_up(incl, d);
       if (lane >= d) incl += y;
     }
-    int run = incl - sum;
+    const int base = incl - sum;
     for (int q = 0; q < per; ++q) {
       const int g = g0 + q;
-      if (g < p.G) {
-        s_pref[g] = run;
-        run += (p.offs[g] - (g ? p.offs[g - 1] : 0) + BM - 1) / BM;
-      }
+      if (g < p.G) s_pref[g + 1] += base;
     }
-    if (tid == 63) s_pref[p.G] = incl;
+    if (tid == 0) s_pref[0] = 0;
   }
   __syncthreads();
+}
+
+// m-grouped: s_pref[g] = number of BM-row tiles of groups < g, from the cumulative group ends.
+template <int BM>
+__device__ __forceinline__ void scan_group_tiles(const GemmArgs& p, int* s_pref, int tid, int lane) {
+  scan_groups(p, s_pref, tid, lane, [](int rows) { return (rows + BM - 1) / BM; });
+}
+
+// k-grouped: a tile of group g costs its number of 128-deep reduction blocks plus a fixed share
+// for the tile switch and the result store; s_pref[g] = that cost summed over groups < g.
+static constexpr int kTileFixedCost = 3;
+__device__ __forceinline__ int k_group_tile_cost(int rows) { return ((rows + 127) >> 7) + kTileFixedCost; }
+__device__ __forceinline__ void scan_group_costs(const GemmArgs& p, int* s_pref, int tid, int lane) {
+  scan_groups(p, s_pref, tid, lane, [](int rows) { return k_group_tile_cost(rows); });
+}
+
+// First logical tile of XCD `x` (x in [0, 8]; x = 8 gives the end of the list).  Dense and
+// m-grouped tiles all cost the same, so the list is cut into eight equal counts.  k-grouped tiles
+// cost in proportion to their group's row count: the list (group-major) is cut where the summed
+// cost reaches x/8 of the total, so that skewed group sizes do not leave most XCDs idle while one
+// works through the large groups.
+template <int MODE>
+__device__ __forceinline__ int xcd_first_tile(const GemmArgs& p, const int* s_pref, int total_tiles, int x) {
+  if (MODE != GEMM_K_GROUPED) {
+    const int per_xcd = (total_tiles + 7) / 8;
+    const int t = x * per_xcd;
+    return t < total_tiles ? t : total_tiles;
+  }
+  if (x <= 0) return 0;
+  if (x >= 8) return total_tiles;
+  const int per_g = p.tiles_a * p.tiles_b;
+  const int64_t pos = (int64_t)s_pref[p.G] * per_g * x / 8;
+  int lo = 0, hi = p.G - 1;  // last g with s_pref[g] * per_g <= pos
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if ((int64_t)s_pref[mid] * per_g <= pos) lo = mid; else hi = mid - 1;
+  }
+  const int cost = s_pref[lo + 1] - s_pref[lo];
+  int idx = (int)((pos - (int64_t)s_pref[lo] * per_g) / cost);
+  if (idx > per_g) idx = per_g;
+  return lo * per_g + idx;
 }
 
 // Geometry of logical tile t; plain per-lane arithmetic (every lane may ask for a different t).

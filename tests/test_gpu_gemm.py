@@ -150,7 +150,17 @@ def test_m_grouped_nt_scattered_rows(sizes, N, K, gemm_kernel):
     assert (out[untouched] == 7.0).all()
 
 
-@pytest.mark.parametrize("sizes,N,K", GROUPED)
+# Skewed group sizes: the weight-gradient tiles are shared out over the XCDs by cost (a tile's
+# reduction length), so the cuts fall inside groups, at empty groups and at the ends of the list.
+SKEWED = [
+    ([0] * 5 + [4096] + [0] * 10 + [130, 1, 1, 1], 512, 512),
+    ([3, 900, 0, 17, 2500, 128, 0, 0, 1, 640] * 7, 256, 256),
+    ([2000], 768, 256),
+    ([1] * 9, 256, 512),
+]
+
+
+@pytest.mark.parametrize("sizes,N,K", GROUPED + SKEWED)
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_k_grouped_wgrad(sizes, N, K, accumulate):
     from pith_train_amd.operators.grouped_linear import k_grouped_fp8_wgrad
