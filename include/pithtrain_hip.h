@@ -81,6 +81,27 @@ int pt_silu_mul_bwd_quant_rowwise_colwise(const void* grad_h, int64_t ld_grad_h,
                                           int64_t half, void* tok_fp8, float* tok_scale,
                                           void* ch_t_fp8, float* ch_scale, const int32_t* valid_rows,
                                           pt_stream_t stream);
+/* The same pair for the clamped SwiGLU of GPT-OSS (interleaved (gate, up) pairs, alpha, limit):
+ * quantises h = clamped_swiglu(gate_up[M,2*half]) (clamped_swiglu.py:18-46) as
+ * fp8cast_rowwise_colwise (deepgemm_quantize.py:204-259) would, without writing h:
+ * tok_fp8[M,half], tok_scale[M,ceil(half/128)], ch_t_fp8[half,M], ch_scale[M/128,half]. */
+int pt_clamped_swiglu_quant_rowwise_colwise(const void* gate_up, int64_t M, int64_t half,
+                                            int64_t ld_gate_up, float alpha, float limit,
+                                            void* tok_fp8, float* tok_scale, void* ch_t_fp8,
+                                            float* ch_scale, const int32_t* valid_rows,
+                                            pt_stream_t stream);
+/* Backward twin: the gradient of gate_up in its interleaved layout (clamped_swiglu.py:49-89) from
+ * grad_h[M,half], rounded to bf16 and quantised to tok_fp8[M,2*half], tok_scale[M,ceil(2*half/128)],
+ * ch_t_fp8[2*half,M], ch_scale[M/128,2*half].  col_sum[M/128, 2*half] (fp32) receives the column
+ * sums of every 128-row tile of the bf16 gradient: summed over a group's tiles (pt_segment_sum
+ * with the group ends divided by 128) they are the bias gradient that _segment_sum_kernel
+ * (indexed_bias_add.py:20-51) computes from the materialised gradient. */
+int pt_clamped_swiglu_bwd_quant_rowwise_colwise(const void* grad_h, int64_t ld_grad_h,
+                                                const void* gate_up, int64_t ld_gate_up, int64_t M,
+                                                int64_t half, float alpha, float limit,
+                                                void* tok_fp8, float* tok_scale, void* ch_t_fp8,
+                                                float* ch_scale, float* col_sum,
+                                                const int32_t* valid_rows, pt_stream_t stream);
 
 /* rowwise(x) + rowwise(x^T): t_fp8[N,M], t_scale[N,ceil(M/128)].
  * fp8cast_rowwise_transpose, deepgemm_quantize.py:429-482 */

@@ -30,6 +30,8 @@ SIGNATURES = {
     "pt_quant_rowwise_colwise_rows": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, P, c_int, P, I32, P]),
     "pt_silu_mul_quant_rowwise_colwise": (c_int, [P, I64, I64, I64, P, P, P, P, P, P]),
     "pt_silu_mul_bwd_quant_rowwise_colwise": (c_int, [P, I64, P, I64, I64, I64, P, P, P, P, P, P]),
+    "pt_clamped_swiglu_quant_rowwise_colwise": (c_int, [P, I64, I64, I64, F, F, P, P, P, P, P, P]),
+    "pt_clamped_swiglu_bwd_quant_rowwise_colwise": (c_int, [P, I64, P, I64, I64, I64, F, F, P, P, P, P, P, P, P]),
     "pt_quant_rowwise_transpose": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, P]),
     "pt_quant_rowwise_blockwise_transpose": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, P]),
     "pt_quant_blockwise_transpose_batched": (c_int, [P, c_int, I64, I64, I64, I64, I64, P, P, P, P, P]),

@@ -68,6 +68,25 @@ __device__ __forceinline__ void silu_mul_b(float d, float g, float u, float& dg,
   dg = __fmul_rn(__fmul_rn(__fmul_rn(d, u), sig), __fsub_rn(__fadd_rn(1.0f, g), silu));
 }
 
+// Clamped SwiGLU on one (gate, up) pair: (clamp(u, -L, L) + 1) * gc * sigmoid(alpha * gc) with
+// gc = min(g, L); the backward masks each gradient where its input was clamped.
+__device__ __forceinline__ float cswiglu_f(float g, float u, float alpha, float limit) {
+  const float gc = fminf(g, limit);
+  const float uc = fminf(fmaxf(u, -limit), limit);
+  return __fmul_rn(__fadd_rn(uc, 1.0f), __fmul_rn(gc, sigmoidf_fast(__fmul_rn(alpha, gc))));
+}
+__device__ __forceinline__ void cswiglu_b(float d, float g, float u, float alpha, float limit, float& dg, float& du) {
+  const float gc = fminf(g, limit);
+  const float uc = fminf(fmaxf(u, -limit), limit);
+  const float ag = __fmul_rn(alpha, gc);
+  const float sig = sigmoidf_fast(ag);
+  const float grad_uc = __fmul_rn(d, __fmul_rn(gc, sig));
+  const float grad_gc = __fmul_rn(__fmul_rn(__fmul_rn(d, __fadd_rn(uc, 1.0f)), sig),
+                                  __fadd_rn(1.0f, __fmul_rn(ag, __fsub_rn(1.0f, sig))));
+  dg = (g <= limit) ? grad_gc : 0.0f;
+  du = (u >= -limit && u <= limit) ? grad_uc : 0.0f;
+}
+
 // ---- storage types: 8-wide vector and scalar load/store with fp32 math ---------------------------
 struct st_bf16 {
   static constexpr int kBytes = 2;

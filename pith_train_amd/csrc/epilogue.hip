@@ -118,22 +118,7 @@ __global__ __launch_bounds__(256) void silu_mul_2d_kernel(Silu2dArgs p) {
 }
 
 // ---- clamped SwiGLU (interleaved gate/up) ---------------------------------------------------------
-__device__ __forceinline__ float cswiglu_f(float g, float u, float alpha, float limit) {
-  const float gc = fminf(g, limit);
-  const float uc = fminf(fmaxf(u, -limit), limit);
-  return (uc + 1.0f) * (gc * sigmoidf_fast(alpha * gc));
-}
-__device__ __forceinline__ void cswiglu_b(float d, float g, float u, float alpha, float limit, float& dg, float& du) {
-  const float gc = fminf(g, limit);
-  const float uc = fminf(fmaxf(u, -limit), limit);
-  const float sig = sigmoidf_fast(alpha * gc);
-  const float glu = gc * sig;
-  const float grad_uc = d * glu;
-  const float grad_gc = d * (uc + 1.0f) * sig * (1.0f + alpha * gc * (1.0f - sig));
-  dg = (g <= limit) ? grad_gc : 0.0f;
-  du = (u >= -limit && u <= limit) ? grad_uc : 0.0f;
-}
-
+// cswiglu_f / cswiglu_b live in common.h (shared with the fused quantisation).
 template <typename S>
 __global__ __launch_bounds__(256) void clamped_swiglu_fwd_kernel(const char* gu, char* out, int64_t n, float alpha, float limit) {
   const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;

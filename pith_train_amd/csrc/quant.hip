@@ -36,6 +36,8 @@ struct QuantArgs {
   const int32_t* row_limit;      // optional device scalar: row tiles at or past *row_limit are skipped (nothing written)
   int64_t ld_t;                  // row pitch of the transposed twin (bytes = elements); M unless it is a column slice
   int64_t bs_ld;                 // row length of the twin's block-scale grid; tiles_m unless it is a column slice
+  float alpha, limit;            // fused clamped SwiGLU: its two constants
+  float* col_sum;                // fused clamped SwiGLU backward: [tiles_m, N] column sums of each 128-row tile
 };
 
 template <typename T> struct Loader;
@@ -103,7 +105,8 @@ template <> struct Frag<float> {
   __device__ __forceinline__ void fence_row(int) {}
 };
 
-enum { PRO_NONE = 0, PRO_SILU_FWD = 1, PRO_SILU_BWD = 2, PRO_SILU_BWD_PAIR = 3 };  // what the tile is computed from
+// what the tile is computed from
+enum { PRO_NONE = 0, PRO_SILU_FWD = 1, PRO_SILU_BWD = 2, PRO_SILU_BWD_PAIR = 3, PRO_CSWIGLU_FWD = 4, PRO_CSWIGLU_BWD = 5 };
 
 // ---- packed-bf16 arithmetic of the interior-tile path -------------------------------------------
 // |x| of a bf16 is its low 15 bits, and for non-negative floats the integer order of the bits is
@@ -140,7 +143,8 @@ __device__ __forceinline__ uint32_t cvt4_e4m3_scaled(uint32_t p01, uint32_t p23,
 // bounds are checked; for bf16 sources it also selects the packed arithmetic above.
 template <typename T, int AM, int BMODE, int BL, int BS, int PRO, bool FULL>
 __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_colmax)[128], float* s_blk, uint8_t* s_t,
-                                                const int tc, const int tr, const int64_t g) {
+                                                [[maybe_unused]] float (*s_colsum)[128], const int tc, const int tr,
+                                                const int64_t g) {
   constexpr bool PK = FULL && std::is_same<T, bf16_tag>::value;  // packed-bf16 arithmetic
   const int t = threadIdx.x;
   const int cc = t & 15, rg = t >> 4, wave = t >> 6, lane = t & 63;
@@ -177,6 +181,48 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
       } else {
         f.zero_row(i);
         f_up.zero_row(i);
+      }
+    }
+  } else if constexpr (PRO == PRO_CSWIGLU_FWD) {
+    // h = clamped SwiGLU of the interleaved (gate, up) pairs of gate_up = x, rounded to bf16:
+    // sixteen consecutive inputs give the thread's eight outputs of a row.
+    const bool col_ok = FULL || col0 < p.N;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (FULL || (col_ok && row0 + i < p.M)) {
+        const char* gp = xb + ((row0 + i) * p.ldx + 2 * col0) * 2;
+        float a[8], b[8], o[8];
+        st_bf16::load8(gp, a);
+        st_bf16::load8(gp + 16, b);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          o[j] = cswiglu_f(a[2 * j], a[2 * j + 1], p.alpha, p.limit);
+          o[4 + j] = cswiglu_f(b[2 * j], b[2 * j + 1], p.alpha, p.limit);
+        }
+        f.w[i][0] = pack_bf16x2(o[0], o[1]); f.w[i][1] = pack_bf16x2(o[2], o[3]);
+        f.w[i][2] = pack_bf16x2(o[4], o[5]); f.w[i][3] = pack_bf16x2(o[6], o[7]);
+      } else {
+        f.zero_row(i);
+      }
+    }
+  } else if constexpr (PRO == PRO_CSWIGLU_BWD) {
+    // The gradient of gate_up = x2 in its own interleaved layout, (dgate, dup) pairs rounded to
+    // bf16, from grad_h = x (one column per pair): four pairs per thread and row.
+    const bool col_ok = FULL || col0 < p.N;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (FULL || (col_ok && row0 + i < p.M)) {
+        const int64_t r = row0 + i;
+        const uint2 dw = *reinterpret_cast<const uint2*>(xb + (r * p.ldx + (col0 >> 1)) * 2);
+        const float d[4] = {bf16_lo(dw.x), bf16_hi(dw.x), bf16_lo(dw.y), bf16_hi(dw.y)};
+        float a[8], o[8];
+        st_bf16::load8((const char*)p.x2 + (r * p.ldx2 + col0) * 2, a);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) cswiglu_b(d[j], a[2 * j], a[2 * j + 1], p.alpha, p.limit, o[2 * j], o[2 * j + 1]);
+        f.w[i][0] = pack_bf16x2(o[0], o[1]); f.w[i][1] = pack_bf16x2(o[2], o[3]);
+        f.w[i][2] = pack_bf16x2(o[4], o[5]); f.w[i][3] = pack_bf16x2(o[6], o[7]);
+      } else {
+        f.zero_row(i);
       }
     }
   } else if constexpr (PRO != PRO_NONE) {
@@ -354,6 +400,20 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
       }
     }
   }
+  if constexpr (PRO == PRO_CSWIGLU_BWD) {
+    // Column sums of the tile's bf16 values (the bias gradient of the projection before the
+    // activation is their sum over a group's tiles): rows of the thread in order, then the four
+    // row groups of a wave pairwise, then the four waves after the barrier.
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float sum = f.get(0, j);
+#pragma unroll
+      for (int i = 1; i < 8; ++i) sum = __fadd_rn(sum, f.get(i, j));
+      sum = __fadd_rn(sum, __shfl_xor(sum, 16));
+      sum = __fadd_rn(sum, __shfl_xor(sum, 32));
+      if (lane < 16) s_colsum[wave][cc * 8 + j] = sum;
+    }
+  }
   float blkmax = 0.f;
   if (AM == A_BLOCK || BMODE == B_BLOCK) {
     float m = rowmax[0];
@@ -365,6 +425,17 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
     if (lane == 0) s_blk[wave] = m;
   }
   __syncthreads();
+  if constexpr (PRO == PRO_CSWIGLU_BWD) {
+    if (rg == 0) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int c = cc * 8 + j;
+        if (FULL || col0 + j < p.N)
+          p.col_sum[(int64_t)tr * p.N + col0 + j] =
+              __fadd_rn(__fadd_rn(s_colsum[0][c], s_colsum[1][c]), __fadd_rn(s_colsum[2][c], s_colsum[3][c]));
+      }
+    }
+  }
   if (BMODE == B_COL) {
     if constexpr (PK) {
       const uint32_t* s_pair = reinterpret_cast<const uint32_t*>(&s_colmax[0][0]);
@@ -519,6 +590,7 @@ void quant_tile_kernel(QuantArgs p) {
   __shared__ float s_colmax[4][128];
   __shared__ float s_blk[4];
   __shared__ __attribute__((aligned(16))) uint8_t s_t[128 * 128];
+  __shared__ float s_colsum[PRO == PRO_CSWIGLU_BWD ? 4 : 1][128];
 
   int64_t bid = blockIdx.x;
   // PRO_SILU_BWD_PAIR: one workgroup produces the dgate tile and its dup twin (half / 128 column
@@ -533,8 +605,8 @@ void quant_tile_kernel(QuantArgs p) {
   // interior tile with every vector access legal (uniform over the workgroup)
   const int64_t n_cols = PRO == PRO_SILU_BWD_PAIR ? p.half : p.N;
   const bool full = (int64_t)tr * 128 + 128 <= p.M && (int64_t)tc * 128 + 128 <= n_cols && p.vec_in && p.vec_out && p.vec_out_t;
-  if (full) quant_tile_body<T, AM, BMODE, BL, BS, PRO, true>(p, s_colmax, s_blk, s_t, tc, tr, g);
-  else      quant_tile_body<T, AM, BMODE, BL, BS, PRO, false>(p, s_colmax, s_blk, s_t, tc, tr, g);
+  if (full) quant_tile_body<T, AM, BMODE, BL, BS, PRO, true>(p, s_colmax, s_blk, s_t, s_colsum, tc, tr, g);
+  else      quant_tile_body<T, AM, BMODE, BL, BS, PRO, false>(p, s_colmax, s_blk, s_t, s_colsum, tc, tr, g);
 }
 
 template <int AM, int BMODE, int BL, int BS>
@@ -556,7 +628,7 @@ static void fill_common(QuantArgs& a, const void* x, int dtype, int64_t M, int64
   a.a_stride_g = 0; a.a_scale_stride_g = 0; a.b_stride_g = 0; a.b_scale_stride_g = 0;
   a.tiles_m = (int32_t)cdiv(M, 128); a.tiles_n = (int32_t)cdiv(N, 128);
   a.offs = nullptr; a.num_groups = 0; a.row_index = nullptr; a.x2 = nullptr; a.ldx2 = 0; a.half = 0;
-  a.row_limit = nullptr; a.ld_t = M; a.bs_ld = a.tiles_m;
+  a.row_limit = nullptr; a.ld_t = M; a.bs_ld = a.tiles_m; a.alpha = 0.f; a.limit = 0.f; a.col_sum = nullptr;
   const int eb = dtype == PT_F32 ? 4 : 2;
   a.vec_in = (N % 8 == 0) && ((ldx * eb) % 16 == 0) && (((uintptr_t)x) % 16 == 0);
   a.vec_out = (N % 8 == 0);
@@ -723,4 +795,42 @@ extern "C" int pt_silu_mul_bwd_quant_rowwise_colwise(const void* grad_h, int64_t
   // with whole 128-column tiles per half, each workgroup makes a dgate tile and its dup twin
   if (half % 128 == 0) return launch_silu_quant<PRO_SILU_BWD_PAIR>(a, (hipStream_t)stream);
   return launch_silu_quant<PRO_SILU_BWD>(a, (hipStream_t)stream);
+}
+
+// ---- clamped SwiGLU (interleaved gate/up) fused into the activation quantisation -----------------
+extern "C" int pt_clamped_swiglu_quant_rowwise_colwise(const void* gate_up, int64_t M, int64_t half, int64_t ld_gate_up,
+                                                       float alpha, float limit, void* tok_fp8, float* tok_scale,
+                                                       void* ch_t_fp8, float* ch_scale, const int32_t* valid_rows,
+                                                       pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && half >= 0 && M % 128 == 0 && ld_gate_up >= 2 * half, "clamped_swiglu_quant: bad shape");
+  if (M == 0 || half == 0) return PT_OK;
+  PT_REQUIRE(gate_up && tok_fp8 && tok_scale && ch_t_fp8 && ch_scale, "clamped_swiglu_quant: null pointer");
+  PT_REQUIRE(half % 8 == 0 && ld_gate_up % 8 == 0 && ((uintptr_t)gate_up) % 16 == 0,
+             "clamped_swiglu_quant: the output width and the row stride must be multiples of 8 elements, the pointer 16-byte aligned");
+  QuantArgs a;
+  fill_common(a, gate_up, PT_BF16, M, half, ld_gate_up);
+  a.half = half; a.row_limit = valid_rows; a.alpha = alpha; a.limit = limit;
+  a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)ch_t_fp8; a.b_scale = ch_scale;
+  return launch_silu_quant<PRO_CSWIGLU_FWD>(a, (hipStream_t)stream);
+}
+
+extern "C" int pt_clamped_swiglu_bwd_quant_rowwise_colwise(const void* grad_h, int64_t ld_grad_h, const void* gate_up,
+                                                           int64_t ld_gate_up, int64_t M, int64_t half, float alpha,
+                                                           float limit, void* tok_fp8, float* tok_scale, void* ch_t_fp8,
+                                                           float* ch_scale, float* col_sum, const int32_t* valid_rows,
+                                                           pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && half >= 0 && M % 128 == 0 && ld_gate_up >= 2 * half && ld_grad_h >= half,
+             "clamped_swiglu_bwd_quant: bad shape");
+  if (M == 0 || half == 0) return PT_OK;
+  PT_REQUIRE(grad_h && gate_up && tok_fp8 && tok_scale && ch_t_fp8 && ch_scale && col_sum, "clamped_swiglu_bwd_quant: null pointer");
+  PT_REQUIRE(half % 4 == 0 && ld_gate_up % 8 == 0 && ld_grad_h % 4 == 0 && ((uintptr_t)gate_up) % 16 == 0 &&
+                 ((uintptr_t)grad_h) % 8 == 0,
+             "clamped_swiglu_bwd_quant: the pair count and the gradient's row stride must be multiples of 4 elements, "
+             "gate_up's row stride a multiple of 8, pointers 8- and 16-byte aligned");
+  QuantArgs a;
+  fill_common(a, grad_h, PT_BF16, M, 2 * half, ld_grad_h);
+  a.half = half; a.x2 = gate_up; a.ldx2 = ld_gate_up; a.row_limit = valid_rows; a.alpha = alpha; a.limit = limit;
+  a.col_sum = col_sum;
+  a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)ch_t_fp8; a.b_scale = ch_scale;
+  return launch_silu_quant<PRO_CSWIGLU_BWD>(a, (hipStream_t)stream);
 }

@@ -150,6 +150,9 @@ class GptOssExperts(nn.Module):
         # extension: the two indexed_bias_add steps happen in the stores of the GEMMs before them
         # (same bits) wherever the shapes and dtypes allow it
         self.fuse_bias = True
+        # extension (needs fuse_bias): the whole block as one autograd node whose quantisation
+        # kernels compute the clamped SwiGLU and its gradient instead of reading them from memory
+        self.fuse_activation = True
 
     def _quantized_weight(self, name: str, weight: torch.Tensor):
         if torch.compiler.is_compiling():
@@ -192,6 +195,12 @@ class GptOssExperts(nn.Module):
         M = x.shape[0] if row_map is None else row_map.shape[0]
         fused = self.bias_fusable(x)
         assert not scatter_output or (fused and row_map is not None), "scatter_output needs row_map and the fused biases"
+        if fused and self.fuse_activation and M % 128 == 0 and self.down_proj.shape[2] % 8 == 0:
+            return fused_experts.FP8ClampedSwiGLUExpertsFunc.apply(
+                x, self.gate_up_proj, self.gate_up_proj_bias, self.down_proj, self.down_proj_bias, grouped_mm_offs,
+                self._quantized_weight("gate_up_proj", self.gate_up_proj), self._quantized_weight("down_proj", self.down_proj),
+                1.702, self.swiglu_limit, row_map, scatter_output,
+            )
         if fused:
             gate_up = self._group_linear(x, self.gate_up_proj, "gate_up_proj", grouped_mm_offs, ks, ks_tensor, None, row_map,
                                          self.gate_up_proj_bias)

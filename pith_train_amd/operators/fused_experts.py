@@ -65,6 +65,45 @@ def silu_mul_bwd_quant(grad_h: torch.Tensor, gate_up: torch.Tensor, grouped_mm_o
     return tok, tok_s, ch_t, ch_s
 
 
+def clamped_swiglu_quant(gate_up: torch.Tensor, alpha: float, limit: float, grouped_mm_offs: torch.Tensor | None = None):
+    """``fp8cast_rowwise_colwise_t(clamped_swiglu(gate_up, alpha, limit))`` in one pass (interleaved
+    (gate, up) pairs, clamped_swiglu.py:95-155); rows limited as in :func:`silu_mul_quant`."""
+    M, two_i = gate_up.shape
+    half = two_i // 2
+    dev = gate_up.device
+    tok = torch.empty((M, half), dtype=FP8, device=dev)
+    tok_s = torch.empty((M, _cdiv(half, 128)), dtype=torch.float32, device=dev)
+    ch_t = torch.empty((half, M), dtype=FP8, device=dev)
+    ch_s = torch.empty((M // 128, half), dtype=torch.float32, device=dev)
+    _lib.call(
+        "pt_clamped_swiglu_quant_rowwise_colwise", gate_up.data_ptr(), M, half, gate_up.stride(0), alpha, limit,
+        tok.data_ptr(), tok_s.data_ptr(), ch_t.data_ptr(), ch_s.data_ptr(), _last(grouped_mm_offs),
+        _lib.stream_ptr(dev),
+    )  # fmt: skip
+    return tok, tok_s, ch_t, ch_s
+
+
+def clamped_swiglu_bwd_quant(grad_h: torch.Tensor, gate_up: torch.Tensor, alpha: float, limit: float,
+                             grouped_mm_offs: torch.Tensor | None = None):
+    """``fp8cast_rowwise_colwise_t`` of the clamped SwiGLU's input gradient in one pass, plus
+    ``col_sum`` ``[M / 128, 2I]`` fp32: the column sums of every 128-row tile of that (bf16-rounded)
+    gradient, from which the bias gradient of the projection before it is summed per group."""
+    M, two_i = gate_up.shape
+    half = two_i // 2
+    dev = gate_up.device
+    tok = torch.empty((M, two_i), dtype=FP8, device=dev)
+    tok_s = torch.empty((M, _cdiv(two_i, 128)), dtype=torch.float32, device=dev)
+    ch_t = torch.empty((two_i, M), dtype=FP8, device=dev)
+    ch_s = torch.empty((M // 128, two_i), dtype=torch.float32, device=dev)
+    col_sum = torch.empty((M // 128, two_i), dtype=torch.float32, device=dev)
+    _lib.call(
+        "pt_clamped_swiglu_bwd_quant_rowwise_colwise", grad_h.data_ptr(), grad_h.stride(0), gate_up.data_ptr(),
+        gate_up.stride(0), M, half, alpha, limit, tok.data_ptr(), tok_s.data_ptr(), ch_t.data_ptr(), ch_s.data_ptr(),
+        col_sum.data_ptr(), _last(grouped_mm_offs), _lib.stream_ptr(dev),
+    )  # fmt: skip
+    return tok, tok_s, ch_t, ch_s, col_sum
+
+
 def supported(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor) -> bool:
     """bf16 activations, half width and hidden size multiples of 8 (16-byte accesses)."""
     half = w_gate_up.shape[1] // 2
@@ -191,3 +230,76 @@ def supported_split(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w
     half = w_gate.shape[1]
     return (x.dtype == torch.bfloat16 and w_gate.shape == w_up.shape and half % 128 == 0
             and w_down.shape[1] % 8 == 0 and w_down.shape[2] == half)
+
+
+class FP8ClampedSwiGLUExpertsFunc(torch.autograd.Function):
+    """The GPT-OSS expert block (models/gpt_oss.py:139-157: gate_up projection + bias, clamped
+    SwiGLU on interleaved pairs, down projection + bias) as one node.  Outputs, input gradient,
+    weight gradients and the down bias gradient have the bits of the composition of
+    ``FP8GroupedLinearFunc`` (biases in the GEMM stores) and ``clamped_swiglu``; the activation
+    and its gradient are never written as bf16 tensors, and the gate_up bias gradient is summed
+    from per-tile column sums that the backward's quantisation produces (fp32, another order of
+    additions than the segmented sum over the materialised gradient: same value up to fp32
+    rounding before the cast to the bias dtype).
+
+    ``row_map`` (int32 ``[M]``, from the scatter): ``x`` is the un-permuted ``[m, K]`` token tensor;
+    with ``scatter_output`` the result comes back un-permuted as well."""
+
+    @staticmethod
+    def forward(ctx, x, w_gate_up, b_gate_up, w_down, b_down, grouped_mm_offs, q_gate_up, q_down, alpha, limit,
+                row_map=None, scatter_output=False):
+        _lib.require_cuda(x)
+        gu_fp8, gu_scale, gu_t_fp8, gu_t_scale = q_gate_up
+        dn_fp8, dn_scale, dn_t_fp8, dn_t_scale = q_down
+        two_i = gu_fp8.shape[1]
+        H = w_down.shape[1]
+        assert not scatter_output or row_map is not None, "scatter_output needs the row map"
+        if row_map is not None:
+            M = row_map.shape[0]
+            x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, row_map)
+        else:
+            M = x.shape[0]
+            x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t(x)
+        gate_up = torch.empty((M, two_i), device=x.device, dtype=x.dtype)
+        m_grouped_fp8_gemm_nt((x_fp8, x_s), (gu_fp8, gu_scale), gate_up, grouped_mm_offs, None,
+                              b_gate_up.detach().contiguous())
+        del x_fp8, x_s
+        h_fp8, h_s, h_ch_t, h_ch_s = clamped_swiglu_quant(gate_up, alpha, limit)
+        out_rows = row_map if scatter_output else None
+        out = torch.empty((x.shape[0] if scatter_output else M, H), device=x.device, dtype=x.dtype)
+        m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, out_rows,
+                              b_down.detach().contiguous())
+        ctx.save_for_backward(gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, grouped_mm_offs, x_ch_t, x_ch_s,
+                              gate_up, h_ch_t, h_ch_s, row_map)
+        ctx.weights = (w_gate_up, w_down)
+        ctx.consts = (float(alpha), float(limit), bool(scatter_output), M, x.shape[0], b_gate_up.dtype, b_down.dtype)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from .indexed_bias_add import _segment_sum_along_rows
+
+        (gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, offs, x_ch_t, x_ch_s, gate_up, h_ch_t, h_ch_s,
+         row_map) = ctx.saved_tensors  # fmt: skip
+        w_gate_up, w_down = ctx.weights
+        alpha, limit, scatter_output, M, rows_x, gu_bias_dtype, dn_bias_dtype = ctx.consts
+        half = gate_up.shape[1] // 2
+        K = gu_t_fp8.shape[1]
+        grad_out = grad_out.contiguous()
+        out_rows = row_map if scatter_output else None
+        if out_rows is not None:
+            dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t_rows(grad_out, out_rows)
+        else:
+            dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t(grad_out)
+        grad_b_down = _segment_sum_along_rows(grad_out, offs, dn_bias_dtype, out_rows)
+        grad_h = torch.empty((M, half), device=grad_out.device, dtype=grad_out.dtype)
+        m_grouped_fp8_gemm_nt((dy_fp8, dy_s), (dn_t_fp8, dn_t_scale), grad_h, offs)
+        schedule_wgrad(w_down, (dy_ch_t, dy_ch_s), (h_ch_t, h_ch_s), offs)
+        del dy_fp8, dy_s
+        dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s, col_sum = clamped_swiglu_bwd_quant(grad_h, gate_up, alpha, limit)
+        # groups are whole 128-row tiles: their ends in tiles index the per-tile column sums
+        grad_b_gate_up = _segment_sum_along_rows(col_sum, offs // 128, gu_bias_dtype)
+        grad_x = torch.empty((rows_x if row_map is not None else M, K), device=grad_out.device, dtype=grad_out.dtype)
+        m_grouped_fp8_gemm_nt((dgu_fp8, dgu_s), (gu_t_fp8, gu_t_scale), grad_x, offs, row_map)
+        schedule_wgrad(w_gate_up, (dgu_ch_t, dgu_ch_s), (x_ch_t, x_ch_s), offs)
+        return grad_x, None, grad_b_gate_up, None, grad_b_down, None, None, None, None, None, None, None

@@ -311,6 +311,7 @@ def test_gpt_oss_bias_folded_into_the_gemm_store_is_bit_identical(kind, E, H, I,
     for fuse_bias, fuse_permute in ((True, True), (False, True), (True, False), (False, False)):
         mod, params = _build(kind, E, H, I, w)
         mod.fuse_bias = fuse_bias
+        mod.fuse_activation = False  # the one-node path has a test of its own below
         FP8WeightCacheControl.step()
         tok = tokens.clone().requires_grad_(True)
         out = forward_stage3(mod, tok, ids.reshape(-1).cuda(), E, fuse_permute=fuse_permute)
@@ -322,3 +323,38 @@ def test_gpt_oss_bias_folded_into_the_gemm_store_is_bit_identical(kind, E, H, I,
         assert torch.equal(res[0][1], other[1]), "token gradient differs"
         for n in res[0][2]:
             assert torch.equal(res[0][2][n], other[2][n]), f"{n} gradient differs"
+
+
+@pytest.mark.parametrize("kind,E,H,I,T,k,zipf", [c for c in CASES if c[0] == "gpt_oss"] + [("gpt_oss", 8, 512, 256, 900, 4, 1.2)])
+def test_gpt_oss_block_as_one_node_matches_the_composition(kind, E, H, I, T, k, zipf):
+    """Clamped SwiGLU and its gradient computed inside the quantisations (one autograd node for
+    the block): output, token gradient, weight gradients and the down bias gradient have the bits
+    of the composition; the gate_up bias gradient is summed from per-tile column sums, in another
+    order of fp32 additions, and may differ by the rounding of that sum to the bias dtype."""
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules.experts import forward_stage3
+
+    ids = OM.make_routing(T, E, k, seed=16, zipf_s=zipf)
+    g = torch.Generator().manual_seed(17)
+    tokens = torch.randn((T * k, H), generator=g).bfloat16().cuda()
+    dy = torch.randn((T * k, H), generator=g).bfloat16().cuda()
+    w = _weights(kind, E, H, I, 18)
+    res = []
+    for fuse_activation, fuse_permute in ((True, True), (False, True), (True, False)):
+        mod, params = _build(kind, E, H, I, w)
+        mod.fuse_activation = fuse_activation
+        FP8WeightCacheControl.step()
+        tok = tokens.clone().requires_grad_(True)
+        out = forward_stage3(mod, tok, ids.reshape(-1).cuda(), E, fuse_permute=fuse_permute)
+        out.backward(dy)
+        res.append((out.detach(), tok.grad, {n: p.grad for n, p in params.items()}))
+    for other in res[1:]:
+        assert torch.equal(res[0][0], other[0]), "forward output differs"
+        assert torch.equal(res[0][1], other[1]), "token gradient differs"
+        for n in res[0][2]:
+            a, b = res[0][2][n], other[2][n]
+            if n == "gate_up_proj_bias":
+                assert (a == b).float().mean() > 0.98, "most sums round to the same bf16 value"
+                torch.testing.assert_close(a.float(), b.float(), rtol=2.0**-7, atol=1e-3 * b.float().abs().max().item())
+            else:
+                assert torch.equal(a, b), f"{n} gradient differs"

@@ -192,3 +192,31 @@ def test_weights_quantised_into_a_fused_operand_equal_the_quantised_concatenatio
     for a, b in zip(got, ref):
         assert a.shape == b.shape
         assert torch.equal(a.view(torch.uint8) if a.dtype != torch.float32 else a, b.view(torch.uint8) if b.dtype != torch.float32 else b)
+
+
+@pytest.mark.parametrize("M,half", [(384, 256), (256, 200), (128, 2880)])
+def test_clamped_swiglu_fused_into_the_quantisation_has_the_bits_of_the_two_steps(M, half):
+    """The GPT-OSS activation computed inside the quantisation kernels: forward bytes and scales,
+    backward bytes and scales equal those of clamped_swiglu (tested against the oracle on its own)
+    followed by the rowwise + colwise quantiser; the per-tile column sums equal the float64 sums
+    of the materialised bf16 gradient to fp32 rounding."""
+    from pith_train_amd.operators import deepgemm_quantize as DQ
+    from pith_train_amd.operators import fused_experts as FE
+    from pith_train_amd.operators.clamped_swiglu import clamped_swiglu
+
+    g = torch.Generator().manual_seed(M + half)
+    gate_up = (torch.randn((M, 2 * half), generator=g) * 4).bfloat16().cuda().requires_grad_(True)
+    grad_h = torch.randn((M, half), generator=g).bfloat16().cuda()
+    h = clamped_swiglu(gate_up, 1.702, 7.0)
+    h.backward(grad_h)
+    u8 = lambda t: t.view(torch.uint8) if t.dtype == torch.float8_e4m3fn else t  # noqa: E731
+    for got, ref in zip(FE.clamped_swiglu_quant(gate_up.detach(), 1.702, 7.0), DQ.fp8cast_rowwise_colwise_t(h.detach())):
+        assert got.shape == ref.shape and torch.equal(u8(got), u8(ref))
+    *quant, col_sum = FE.clamped_swiglu_bwd_quant(grad_h, gate_up.detach(), 1.702, 7.0)
+    for got, ref in zip(quant, DQ.fp8cast_rowwise_colwise_t(gate_up.grad)):
+        assert got.shape == ref.shape and torch.equal(u8(got), u8(ref))
+    tiles = gate_up.grad.double().reshape(M // 128, 128, 2 * half)
+    want, mag = tiles.sum(1), tiles.abs().sum(1)
+    assert col_sum.shape == want.shape
+    assert ((col_sum.double() - want).abs() <= 1e-6 * mag + 1e-30).all()
+    assert (gate_up.grad == 0).any() and (gate_up.grad != 0).any()  # both sides of the clamps occur
