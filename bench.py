@@ -135,7 +135,7 @@ class GemmTimer:
     NAMES = ("pt_gemm_m_grouped_nt", "pt_gemm_m_grouped_nt_scatter", "pt_gemm_m_grouped_nt_bias",
              "pt_gemm_m_grouped_nt_scatter_bias", "pt_gemm_k_grouped_wgrad",
              "pt_gemm_k_grouped_wgrad_ld",
-             "pt_gemm_nt_dense")
+             "pt_gemm_nt_dense", "pt_gemm_nt_dense_splitk")
 
     def __init__(self):
         self.records = []
@@ -157,7 +157,8 @@ class GemmTimer:
                 orig(name, *args)
                 b.record()
                 # rows x columns x reduction as the entry point takes them (the three int64 sizes)
-                sizes = {"pt_gemm_nt_dense": args[6:9], "pt_gemm_k_grouped_wgrad": args[9:12],
+                sizes = {"pt_gemm_nt_dense": args[6:9], "pt_gemm_nt_dense_splitk": args[7:10],
+                         "pt_gemm_k_grouped_wgrad": args[9:12],
                          "pt_gemm_k_grouped_wgrad_ld": args[11:14]}.get(name, args[8:11])
                 timer.records.append((name, a, b, "x".join(str(int(v)) for v in sizes)))
             else:
@@ -188,7 +189,7 @@ class GemmTimer:
         rep = {}
         for (name, shape), (ms, n) in out.items():
             m, nn, k = (int(v) for v in shape.split("x"))
-            if name == "pt_gemm_nt_dense":
+            if name.startswith("pt_gemm_nt_dense"):  # (the split form's slab traffic is not algorithmic)
                 flop = 2.0 * m * nn * k
                 byts = m * k * (1 + 4 / 128) + nn * k * (1 + 4 / 16384) + 2.0 * m * nn
             else:

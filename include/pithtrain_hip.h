@@ -146,6 +146,16 @@ int pt_quant_blockwise_transpose_batched_into(const void* x, int dtype, int64_t 
 int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const void* b_fp8,
                      const float* b_scale, void* out, int out_dtype, int64_t M, int64_t N,
                      int64_t K, pt_stream_t stream);
+/* Split-K form of pt_gemm_nt_dense for outputs with too few 256 x 256 tiles to fill the GPU (the
+ * weight gradient of a dense linear, linear.py:61-83: M, N = weight dims, K = tokens): the
+ * reduction is cut into `splits` ranges of split_len (a multiple of 128), range s is reduced into
+ * the fp32 slab partial[s] ([splits, M, N], caller-provided), and pt_sum_partials adds the slabs
+ * in the order of s and stores the sum as out_dtype (n = M * N, a multiple of 8). */
+int pt_gemm_nt_dense_splitk(const void* a_fp8, const float* a_scale, const void* b_fp8,
+                            const float* b_scale, float* partial, int32_t splits, int64_t split_len,
+                            int64_t M, int64_t N, int64_t K, pt_stream_t stream);
+int pt_sum_partials(const float* partial, int32_t splits, int64_t n, void* out, int out_dtype,
+                    pt_stream_t stream);
 
 /* Rows [offs[g-1], offs[g]) of a[M,K] use b[g] of b[G,N,K]; every offs[g] is a multiple of 128.
  * Rows at or past offs[G-1] are not written.  out bf16 [M,N].

@@ -38,6 +38,8 @@ SIGNATURES = {
     "pt_quant_blockwise_transpose_batched_into": (c_int, [P, c_int, I64, I64, I64, I64, I64, P, I64, P, I64, P, I64, I64, P, I64,
                                                           I64, P]),
     "pt_gemm_nt_dense": (c_int, [P, P, P, P, P, c_int, I64, I64, I64, P]),
+    "pt_gemm_nt_dense_splitk": (c_int, [P, P, P, P, P, I32, I64, I64, I64, I64, P]),
+    "pt_sum_partials": (c_int, [P, I32, I64, P, c_int, P]),
     "pt_gemm_m_grouped_nt": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P]),
     "pt_gemm_m_grouped_nt_bias": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, P]),
     "pt_gemm_m_grouped_nt_scatter_bias": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, I64, P, P]),

@@ -87,7 +87,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_nt_kernel(GemmArgs p)
     const int ta = (int)(idx % p.tiles_a), tb = (int)(idx / p.tiles_a);
     a_row0 = (int64_t)ta * BM; b_row0 = (int64_t)tb * BN;
     a_lim = p.rows_a; b_lim = p.rows_b;
-    k_begin = g == 0 ? 0 : p.offs[g - 1]; k_end = p.offs[g]; kb0 = k_begin >> 7;
+    k_begin = g == 0 ? 0 : k_group_end(p, g - 1); k_end = k_group_end(p, g); kb0 = k_begin >> 7;
     outp += (int64_t)g * p.out_stride_g * (p.out_dtype == PT_F32 ? 4 : 2);
   }
   const int nk = (int)((k_end - k_begin + 127) >> 7);
@@ -343,6 +343,66 @@ extern "C" int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const v
   g.tiles_a = (int)cdiv(M, 128); g.tiles_b = (int)cdiv(N, 128);
   g.total_tiles = (int64_t)g.tiles_a * g.tiles_b;
   return dispatch_gemm(g, (hipStream_t)stream);
+}
+
+// ---- split-K: a dense GEMM whose output has too few tiles to fill the GPU ------------------------
+// The reduction is cut into `splits` ranges of split_len (a multiple of 128, so every range starts
+// on a scale block); range s is computed like a group of the k-grouped mode into the fp32 slab
+// partial[s] (M x N), and pt_sum_partials adds the slabs in the order of s.
+extern "C" int pt_gemm_nt_dense_splitk(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
+                                       float* partial, int32_t splits, int64_t split_len, int64_t M, int64_t N, int64_t K,
+                                       pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_nt_dense_splitk: negative size");
+  if (M == 0 || N == 0) return PT_OK;
+  PT_REQUIRE(K > 0 && K % 16 == 0, "gemm_nt_dense_splitk: K=%lld must be a positive multiple of 16", (long long)K);
+  PT_REQUIRE(splits >= 1 && split_len > 0 && split_len % 128 == 0 && (int64_t)splits * split_len >= K &&
+                 (int64_t)(splits - 1) * split_len < K,
+             "gemm_nt_dense_splitk: %d ranges of %lld (a multiple of 128) must cover K=%lld with none empty", splits,
+             (long long)split_len, (long long)K);
+  PT_REQUIRE(a_fp8 && a_scale && b_fp8 && b_scale && partial && al16(a_fp8) && al16(b_fp8),
+             "gemm_nt_dense_splitk: null or misaligned pointer");
+  const int64_t KB = cdiv(K, 128);
+  GemmArgs g = {};
+  g.a = (const uint8_t*)a_fp8; g.lda = K; g.b = (const uint8_t*)b_fp8; g.ldb = K;
+  g.sa = a_scale; g.sa_rs = KB; g.sa_ks = 1; g.sa_shift = 0;
+  g.sb = b_scale; g.sb_rs = KB; g.sb_ks = 1; g.sb_shift = 7;
+  g.out = partial; g.ldo = N; g.out_dtype = PT_F32; g.accumulate = 0;
+  g.rows_a = M; g.rows_b = N; g.red = K; g.mode = GEMM_K_GROUPED; g.offs = nullptr; g.G = splits; g.split_len = split_len;
+  g.out_stride_g = M * N;
+  g.a_bytes = M * g.lda; g.b_bytes = N * g.ldb; g.sa_bytes = M * KB * 4; g.sb_bytes = cdiv(N, 128) * KB * 4;
+  g.tiles_a = (int)cdiv(M, 128); g.tiles_b = (int)cdiv(N, 128);
+  g.total_tiles = (int64_t)g.tiles_a * g.tiles_b * splits;
+  return dispatch_gemm(g, (hipStream_t)stream);
+}
+
+namespace pt {
+template <typename S>
+__global__ __launch_bounds__(256) void sum_partials_kernel(const float* partial, int splits, int64_t n, char* out) {
+  const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;  // n is a multiple of 8
+  if (i0 >= n) return;
+  float acc[8];
+  st_f32::load8(partial + i0, acc);
+  for (int s = 1; s < splits; ++s) {
+    float v[8];
+    st_f32::load8(partial + (int64_t)s * n + i0, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] += v[j];
+  }
+  S::store8(out + i0 * S::kBytes, acc);
+}
+}  // namespace pt
+
+extern "C" int pt_sum_partials(const float* partial, int32_t splits, int64_t n, void* out, int out_dtype, pt_stream_t stream) {
+  PT_REQUIRE(splits >= 1 && n >= 0, "sum_partials: bad sizes");
+  if (n == 0) return PT_OK;
+  PT_REQUIRE(partial && out && al16(partial) && al16(out) && n % 8 == 0, "sum_partials: null or misaligned pointer, or n not a multiple of 8");
+  PT_REQUIRE(out_dtype == PT_BF16 || out_dtype == PT_F32, "sum_partials: out_dtype must be bf16 or fp32");
+  const int64_t blocks = cdiv(n, 2048);
+  PT_REQUIRE(blocks < (1ll << 31), "sum_partials: too many elements");
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == PT_BF16) hipLaunchKernelGGL((sum_partials_kernel<st_bf16>), dim3((unsigned)blocks), dim3(256), 0, st, partial, splits, n, (char*)out);
+  else hipLaunchKernelGGL((sum_partials_kernel<st_f32>), dim3((unsigned)blocks), dim3(256), 0, st, partial, splits, n, (char*)out);
+  return check_launch("sum_partials_kernel");
 }
 
 static int gemm_m_grouped_impl(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale, void* out,

@@ -23,7 +23,15 @@ struct GemmArgs {
   const int32_t* out_row_index;           // m-grouped only: output row of result row r (negative: dropped); null = identity
   int64_t out_rows;                       // rows of the output when out_row_index is given
   const void* bias;                       // m-grouped only: [G, rows_b] in the output's type, row g added to the rows of group g
+  int64_t split_len;                      // k-grouped with offs == null: group g reduces over [g, g + 1) * split_len (split-K)
 };
+
+// End of group g's reduction range in the k-grouped mode (its start is the end of group g - 1).
+__device__ __forceinline__ int k_group_end(const GemmArgs& p, int g) {
+  if (p.offs) return p.offs[g];
+  const int64_t e = (int64_t)(g + 1) * p.split_len;
+  return (int)(e < p.red ? e : p.red);
+}
 
 
 // persistent kernel with the two-phase main loop (gemm_persistent.hip); variant selects the wave layout

@@ -192,20 +192,20 @@ __device__ __forceinline__ void mfma_sel(const v8i& a, const v8i& b, v16f& c, in
 
 // s_pref[g] = sum of weight(g') over groups g' < g (s_pref[G] = the total); computed by the first
 // wave, followed by a workgroup barrier.
-template <class W>
-__device__ __forceinline__ void scan_groups(const GemmArgs& p, int* s_pref, int tid, int lane, W weight) {
+template <class E, class W>
+__device__ __forceinline__ void scan_groups(const GemmArgs& p, int* s_pref, int tid, int lane, E end_of, W weight) {
   if (tid < 64) {
     // Lane l owns groups [l * per, (l + 1) * per): one global read per group, running sums kept in
     // LDS, then the lanes' totals are scanned and added to each lane's own entries.
     const int per = (p.G + 63) / 64;
     const int g0 = tid * per;
-    int prev = (g0 > 0 && g0 <= p.G) ? p.offs[g0 - 1] : 0;
+    int prev = (g0 > 0 && g0 <= p.G) ? end_of(g0 - 1) : 0;
     int sum = 0;
 #pragma unroll 4
     for (int q = 0; q < per; ++q) {
       const int g = g0 + q;
       if (g < p.G) {
-        const int cur = p.offs[g];
+        const int cur = end_of(g);
         sum += weight(cur - prev);
         prev = cur;
         s_pref[g + 1] = sum;
@@ -230,7 +230,7 @@ __device__ __forceinline__ void scan_groups(const GemmArgs& p, int* s_pref, int 
 // m-grouped: s_pref[g] = number of BM-row tiles of groups < g, from the cumulative group ends.
 template <int BM>
 __device__ __forceinline__ void scan_group_tiles(const GemmArgs& p, int* s_pref, int tid, int lane) {
-  scan_groups(p, s_pref, tid, lane, [](int rows) { return (rows + BM - 1) / BM; });
+  scan_groups(p, s_pref, tid, lane, [&](int g) { return p.offs[g]; }, [](int rows) { return (rows + BM - 1) / BM; });
 }
 
 // k-grouped: a tile of group g costs its number of 128-deep reduction blocks plus a fixed share
@@ -238,7 +238,7 @@ __device__ __forceinline__ void scan_group_tiles(const GemmArgs& p, int* s_pref,
 static constexpr int kTileFixedCost = 3;
 __device__ __forceinline__ int k_group_tile_cost(int rows) { return ((rows + 127) >> 7) + kTileFixedCost; }
 __device__ __forceinline__ void scan_group_costs(const GemmArgs& p, int* s_pref, int tid, int lane) {
-  scan_groups(p, s_pref, tid, lane, [](int rows) { return k_group_tile_cost(rows); });
+  scan_groups(p, s_pref, tid, lane, [&](int g) { return k_group_end(p, g); }, [](int rows) { return k_group_tile_cost(rows); });
 }
 
 // First logical tile of XCD `x` (x in [0, 8]; x = 8 gives the end of the list).  Dense and
@@ -313,7 +313,7 @@ __device__ __forceinline__ void decode_tile(const GemmArgs& p, const int* s_pref
     T.g = g;
     T.a_row0 = (idx % p.tiles_a) * BM; T.b_row0 = (idx / p.tiles_a) * BN;
     T.a_lim = (int)p.rows_a; T.b_lim = (int)p.rows_b;
-    T.k_begin = g ? p.offs[g - 1] : 0; T.k_len = p.offs[g] - T.k_begin; T.kb0 = T.k_begin >> 7;
+    T.k_begin = g ? k_group_end(p, g - 1) : 0; T.k_len = k_group_end(p, g) - T.k_begin; T.kb0 = T.k_begin >> 7;
   }
 }
 

@@ -26,6 +26,24 @@ from .deepgemm_quantize import (
 ARCH_MAJOR = 9
 
 
+_WORKGROUPS = 256  # one persistent workgroup per compute unit of the MI355X
+
+
+def _split_k(m: int, n: int, k: int):
+    """(splits, split_len) for out[m, n] = a[m, k] @ b[n, k].T.  An output with fewer 256 x 256
+    tiles than the GPU has compute units (the weight gradient of a dense linear: small output,
+    reduction over all tokens) leaves most of them idle, so its reduction is cut into ranges that
+    are computed side by side into fp32 slabs and summed afterwards.  Ranges are multiples of 128
+    (whole scale blocks) and at least 1024 long, so the extra slab traffic stays small."""
+    tiles = -(-m // 256) * -(-n // 256)
+    if tiles * 2 > _WORKGROUPS or k < 2048 or (m * n) % 8:
+        return 1, k
+    want = min(_WORKGROUPS // tiles, k // 1024)
+    split_len = (-(-k // want) + 127) // 128 * 128
+    splits = -(-k // split_len)
+    return (splits, split_len) if splits > 1 else (1, k)
+
+
 def _fp8_gemm_nt(a_fp8, a_scale, b_fp8, b_scale, m: int, n: int, device, dtype) -> torch.Tensor:
     """out[m, n] = a @ b.T; a: 1x128 scales, b: 128x128 scales."""
     k = a_fp8.shape[1]
@@ -39,6 +57,16 @@ def _fp8_gemm_nt(a_fp8, a_scale, b_fp8, b_scale, m: int, n: int, device, dtype) 
         k += pad
     out_dtype = dtype if dtype in (torch.bfloat16, torch.float32) else torch.float32
     out = torch.empty((m, n), device=device, dtype=out_dtype)
+    splits, split_len = _split_k(m, n, k)
+    if splits > 1:
+        partial = torch.empty((splits, m, n), device=device, dtype=torch.float32)
+        _lib.call(
+            "pt_gemm_nt_dense_splitk", a_fp8.data_ptr(), a_scale.data_ptr(), b_fp8.data_ptr(), b_scale.data_ptr(),
+            partial.data_ptr(), splits, split_len, m, n, k, _lib.stream_ptr(device),
+        )  # fmt: skip
+        _lib.call("pt_sum_partials", partial.data_ptr(), splits, m * n, out.data_ptr(), _lib.dtype_code(out_dtype),
+                  _lib.stream_ptr(device))  # fmt: skip
+        return out if out_dtype == dtype else out.to(dtype)
     _lib.call(
         "pt_gemm_nt_dense", a_fp8.data_ptr(), a_scale.data_ptr(), b_fp8.data_ptr(),
         b_scale.data_ptr(), out.data_ptr(), _lib.dtype_code(out_dtype), m, n, k,

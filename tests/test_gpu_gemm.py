@@ -61,6 +61,36 @@ def test_dense_nt(M, N, K):
     _check(out32, ref, f"dense fp32 {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("M,N,K", [(512, 256, 4096), (300, 200, 4000), (128, 128, 20000), (256, 1024, 2048)])
+def test_dense_nt_with_the_reduction_split_over_workgroups(M, N, K):
+    """Small outputs with a long reduction (a dense weight gradient) are computed as several
+    ranges of the reduction side by side and summed: same result within the GEMM tolerance, through
+    the operator's own rule and through the C-ABI with other range lengths (ragged last range,
+    one range)."""
+    from pith_train_amd import _lib
+    from pith_train_amd.operators.linear import _fp8_gemm_nt, _split_k
+
+    x, w = _rand((M, K), M + K + 2), _rand((N, K), N + K + 3, 0.02)
+    a, sa, _, _ = Q.fp8cast_rowwise_transpose(x)
+    b, sb, _, _ = Q.fp8cast_blockwise_transpose(w)
+    ref = G.gemm_nt_dense(a, sa, b, sb, torch.float64)
+    assert _split_k(M, N, K)[0] > 1, "the case is meant to take the split path"
+    ad, sad, bd, sbd = a.cuda(), sa.cuda(), b.cuda(), sb.cuda()
+    _check(_fp8_gemm_nt(ad, sad, bd, sbd, M, N, "cuda", torch.bfloat16), ref, f"split dense {M}x{N}x{K}")
+    for split_len in (128, 640, (K + 127) // 128 * 128):
+        splits = (K + split_len - 1) // split_len
+        partial = torch.full((splits, M, N), float("nan"), device="cuda")
+        _lib.call("pt_gemm_nt_dense_splitk", ad.data_ptr(), sad.data_ptr(), bd.data_ptr(), sbd.data_ptr(), partial.data_ptr(),
+                  splits, split_len, M, N, K, _lib.stream_ptr("cuda"))
+        for dt in (torch.float32, torch.bfloat16):
+            out = torch.empty((M, N), device="cuda", dtype=dt)
+            _lib.call("pt_sum_partials", partial.data_ptr(), splits, M * N, out.data_ptr(), _lib.dtype_code(dt),
+                      _lib.stream_ptr("cuda"))
+            _check(out, ref, f"split dense {M}x{N}x{K} in {splits} ranges of {split_len} as {dt}")
+        # the slabs are the partial products of their ranges: they add up in float64 as well
+        _check(partial.double().sum(0), ref, "slabs")
+
+
 def test_dense_scale_extremes():
     """Rows with very different magnitudes: the E8M0 exponents given to the MFMA must be per row."""
     from pith_train_amd.operators.linear import _fp8_gemm_nt
