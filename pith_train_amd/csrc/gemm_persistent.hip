@@ -219,13 +219,28 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
+    // The two waves of a SIMD (w and w + NW/2) run half a block apart: the later one keeps the
+    // second MFMA step of a block until after the next block's barrier, so its MFMAs run while the
+    // earlier wave reads its fragments and its own reads run under the earlier wave's MFMAs.  (It
+    // holds the step's fragments over the barrier, which it did anyway; the ring slot is free
+    // once they are in registers.)  The step still pending when the tile ends runs before the
+    // epilogue.
+    const bool late = wave >= NW / 2;
+    v8i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+    int sca[TM], scb[TN];
+    auto mfma_step = [&](const v8i* af, const v8i* bf) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf[j], acc[i][j], 0, 0, 0, sca[i], 0, scb[j]);
+    };
 #pragma unroll 1
     for (int it = 0; it < nk; ++it, ++gb) {
       wait_stage(gb);
       __syncthreads();  // everybody's share of stage gb has landed
-      v8i fa0[TM], fb0[TN], fa1[TM], fb1[TN];
-      int sca[TM], scb[TN];
       if (wave_active) {
+        if (late && it > 0) mfma_step(fa1, fb1);  // second step of the block before
         const float* scA = sc_lds + (gb % NS) * (BM + BN);
         const float* scB = scA + BM;
 #pragma unroll
@@ -234,24 +249,15 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
         for (int j = 0; j < TN; ++j) scb[j] = (int)(__float_as_uint(scB[wn0 + j * 32 + (lane & 31)]) >> 23);
         read_frags(gb, 0, fa0, fb0);
         read_frags(gb, 1, fa1, fb1);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa0[i], fb0[j], acc[i][j], 0, 0, 0, sca[i], 0, scb[j]);
+        mfma_step(fa0, fb0);
       }
       // Every wave has pulled both steps' fragments of stage gb into registers: its ring slot can
       // be refilled now, half a stage before the next barrier (the loads get 1.5 stages to land).
       __syncthreads();
       issue_stage();
-      if (wave_active) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa1[i], fb1[j], acc[i][j], 0, 0, 0, sca[i], 0, scb[j]);
-      }
+      if (wave_active && !late) mfma_step(fa1, fb1);
     }
+    if (wave_active && late && nk > 0) mfma_step(fa1, fb1);
 
     // ---- epilogue ----
     if (!wave_active) continue;
