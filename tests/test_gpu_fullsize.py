@@ -100,3 +100,33 @@ def test_full_size_scatter_covers_every_row_once_and_quant_round_trips():
     # an e4m3 value is within 2**-4 relative (half a step of the 3-bit mantissa) or half a subnormal step
     bound = xp.float().abs().view(xp.shape[0], -1, 128) * 2.0**-4 + s.unsqueeze(-1) * 2.0**-10
     assert (err <= bound).all()
+
+
+def test_full_size_dense_weight_gradient_split_over_the_reduction_matches_the_single_pass():
+    """The k/v and q projections' weight gradients at 32768 tokens (512 x 2048 and 4096 x 2048
+    outputs, reduction 32768): the operator cuts the reduction into ranges; the sum of the ranges
+    equals the single-pass kernel's result up to fp32 summation order, and sampled output rows
+    equal the oracle's float64 product."""
+    from oracle import fp8 as Q
+    from pith_train_amd import _lib
+    from pith_train_amd.operators import deepgemm_quantize as DQ
+    from pith_train_amd.operators.linear import _fp8_gemm_nt, _split_k
+
+    tokens = 32768
+    g = torch.Generator().manual_seed(3)
+    for n_out, n_in in ((512, 2048), (4096, 2048)):
+        grad = torch.randn((tokens, n_out), generator=g).bfloat16().cuda()
+        x = torch.randn((tokens, n_in), generator=g).bfloat16().cuda()
+        _, _, gt, gt_s = DQ.fp8cast_rowwise_transpose(grad)            # grad^T rows, 1x128 scales
+        _, _, xt, xt_s = DQ.fp8cast_rowwise_blockwise_transpose(x)     # x^T, 128x128 scales
+        assert _split_k(n_out, n_in, tokens)[0] > 1
+        split = _fp8_gemm_nt(gt, gt_s, xt, xt_s, n_out, n_in, "cuda", torch.float32)
+        single = torch.empty((n_out, n_in), device="cuda", dtype=torch.float32)
+        _lib.call("pt_gemm_nt_dense", gt.data_ptr(), gt_s.data_ptr(), xt.data_ptr(), xt_s.data_ptr(), single.data_ptr(),
+                  _lib.dtype_code(torch.float32), n_out, n_in, tokens, _lib.stream_ptr("cuda"))
+        scale = single.abs().mean().item()
+        assert (split - single).abs().max().item() <= 1e-4 * scale * 50, "more than fp32 reordering noise"
+        rows = torch.tensor([0, 127, 128, n_out - 1])
+        ref = G.gemm_nt_dense(gt[rows].cpu(), gt_s[rows].cpu(), xt.cpu(), xt_s.cpu(), torch.float64)
+        got = split[rows].cpu().double()
+        assert ((got - ref).abs() <= 1e-2 * ref.abs() + 1e-2 * ref.pow(2).mean().sqrt()).all()
