@@ -271,12 +271,10 @@ __device__ __forceinline__ int xcd_first_tile(const GemmArgs& p, const int* s_pr
 // Geometry of logical tile t; plain per-lane arithmetic (every lane may ask for a different t).
 template <int MODE, int BM, int BN>
 __device__ __forceinline__ void decode_tile(const GemmArgs& p, const int* s_pref, int t, Tile& T) {
-  if (MODE == GEMM_DENSE) {
-    T.g = 0;
-    // The 32 CUs of an XCD work on 32 consecutive logical tiles at a time; laying those out as
-    // a 4 x 8 block of the output makes them share 4 a-tiles and 8 b-tiles in that XCD's L2
-    // instead of 32 a-tiles and 1 b-tile.
-    int ta, tb;
+  // The 32 CUs of an XCD work on 32 consecutive logical tiles at a time; laying those out as a
+  // 4 x 8 block of the output makes them share 4 a-tiles and 8 b-tiles in that XCD's L2 instead
+  // of 32 a-tiles and 1 b-tile.
+  auto blocked = [&](int t, int& ta, int& tb) {
     const int full_a = p.tiles_a & ~3, full_b = p.tiles_b & ~7;
     const int nblk = (full_a >> 2) * (full_b >> 3);
     if (t < nblk * 32) {
@@ -289,6 +287,11 @@ __device__ __forceinline__ void decode_tile(const GemmArgs& p, const int* s_pref
       if (r < fringe_b * p.tiles_a) { ta = r % p.tiles_a; tb = full_b + r / p.tiles_a; }
       else { const int r2 = r - fringe_b * p.tiles_a; ta = full_a + r2 % (p.tiles_a - full_a); tb = r2 / (p.tiles_a - full_a); }
     }
+  };
+  if (MODE == GEMM_DENSE) {
+    T.g = 0;
+    int ta, tb;
+    blocked(t, ta, tb);
     T.a_row0 = ta * BM; T.b_row0 = tb * BN;
     T.a_lim = (int)p.rows_a; T.b_lim = (int)p.rows_b; T.k_begin = 0; T.k_len = (int)p.red; T.kb0 = 0;
   } else if (MODE == GEMM_M_GROUPED) {
@@ -311,7 +314,9 @@ __device__ __forceinline__ void decode_tile(const GemmArgs& p, const int* s_pref
     const int g = t / per_g;
     const int idx = t % per_g;
     T.g = g;
-    T.a_row0 = (idx % p.tiles_a) * BM; T.b_row0 = (idx / p.tiles_a) * BN;
+    int ta = idx % p.tiles_a, tb = idx / p.tiles_a;
+    if (!p.offs) blocked(idx, ta, tb);  // split-K of a dense product: the dense order inside every range
+    T.a_row0 = ta * BM; T.b_row0 = tb * BN;
     T.a_lim = (int)p.rows_a; T.b_lim = (int)p.rows_b;
     T.k_begin = g ? k_group_end(p, g - 1) : 0; T.k_len = k_group_end(p, g) - T.k_begin; T.kb0 = T.k_begin >> 7;
   }
