@@ -55,9 +55,9 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_persistent_kern
   }
   const int xcd = blockIdx.x & 7;
   // lanes 0 and 1 find the two ends of this XCD's share of the list side by side
-  const int t_cut = xcd_first_tile<MODE>(p, s_pref, total_tiles, xcd + (lane & 1));
-  const int t_end = __builtin_amdgcn_readlane(t_cut, 1);
   const int t_step = gridDim.x >> 3;
+  const int t_cut = xcd_first_tile<MODE>(p, s_pref, total_tiles, xcd + (lane & 1), t_step);
+  const int t_end = __builtin_amdgcn_readlane(t_cut, 1);
   const int t_first = __builtin_amdgcn_readlane(t_cut, 0) + (blockIdx.x >> 3);
 
   auto decode_any = [&](int t, Tile& T) { decode_tile<MODE, BM, BN>(p, s_pref, t, T); };

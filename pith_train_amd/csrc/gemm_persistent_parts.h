@@ -199,16 +199,36 @@ __device__ __forceinline__ void scan_groups(const GemmArgs& p, int* s_pref, int 
     // LDS, then the lanes' totals are scanned and added to each lane's own entries.
     const int per = (p.G + 63) / 64;
     const int g0 = tid * per;
-    int prev = (g0 > 0 && g0 <= p.G) ? end_of(g0 - 1) : 0;
     int sum = 0;
-#pragma unroll 4
-    for (int q = 0; q < per; ++q) {
-      const int g = g0 + q;
-      if (g < p.G) {
-        const int cur = end_of(g);
-        sum += weight(cur - prev);
-        prev = cur;
-        s_pref[g + 1] = sum;
+    if (per <= 4) {
+      // up to 256 groups: the lane's five group ends are requested together (one memory latency)
+      const int last = p.G - 1;
+      int e[5];
+#pragma unroll
+      for (int q = 0; q < 5; ++q) {
+        int g = g0 - 1 + q;
+        g = g < 0 ? 0 : (g > last ? last : g);
+        e[q] = end_of(g);
+      }
+      if (g0 == 0) e[0] = 0;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int g = g0 + q;
+        if (q < per && g < p.G) {
+          sum += weight(e[q + 1] - e[q]);
+          s_pref[g + 1] = sum;
+        }
+      }
+    } else {
+      int prev = (g0 > 0 && g0 <= p.G) ? end_of(g0 - 1) : 0;
+      for (int q = 0; q < per; ++q) {
+        const int g = g0 + q;
+        if (g < p.G) {
+          const int cur = end_of(g);
+          sum += weight(cur - prev);
+          prev = cur;
+          s_pref[g + 1] = sum;
+        }
       }
     }
     int incl = sum;
@@ -245,9 +265,10 @@ __device__ __forceinline__ void scan_group_costs(const GemmArgs& p, int* s_pref,
 // m-grouped tiles all cost the same, so the list is cut into eight equal counts.  k-grouped tiles
 // cost in proportion to their group's row count: the list (group-major) is cut where the summed
 // cost reaches x/8 of the total, so that skewed group sizes do not leave most XCDs idle while one
-// works through the large groups.
+// works through the large groups.  Cuts are rounded to multiples of `round`, the number of
+// workgroups per XCD.
 template <int MODE>
-__device__ __forceinline__ int xcd_first_tile(const GemmArgs& p, const int* s_pref, int total_tiles, int x) {
+__device__ __forceinline__ int xcd_first_tile(const GemmArgs& p, const int* s_pref, int total_tiles, int x, int round) {
   if (MODE != GEMM_K_GROUPED) {
     const int per_xcd = (total_tiles + 7) / 8;
     const int t = x * per_xcd;
@@ -265,7 +286,10 @@ __device__ __forceinline__ int xcd_first_tile(const GemmArgs& p, const int* s_pr
   const int cost = s_pref[lo + 1] - s_pref[lo];
   int idx = (int)((pos - (int64_t)s_pref[lo] * per_g) / cost);
   if (idx > per_g) idx = per_g;
-  return lo * per_g + idx;
+  // whole rounds of the XCD's workgroups: a cut a few tiles past a multiple of `round` would
+  // leave most of them idle during one more round
+  const int t = (lo * per_g + idx + (round >> 1)) / round * round;
+  return t < total_tiles ? t : total_tiles;
 }
 
 // Geometry of logical tile t; plain per-lane arithmetic (every lane may ask for a different t).
