@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 # Average HBM bytes moved by one GEMM launch (fetch + write), from the FETCH_SIZE / WRITE_SIZE
 # counter runs summarised under profiles/ (scaled by the same counters' readings for a plain copy
 # of known size).  None for a workload that has no counter run.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-30b-a3b-moe": 795e6}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-30b-a3b-moe": 793e6}
 
 WORKLOADS = {
     # name: (kind, hidden, intermediate, experts, top_k, tokens, zipf)
