@@ -190,8 +190,8 @@ __device__ __forceinline__ void mfma_sel(const v8i& a, const v8i& b, v16f& c, in
 #undef PT_MFMA_TEXT
 }
 
-// s_pref[g] = sum of weight(g') over groups g' < g (s_pref[G] = the total); computed by the first
-// wave, followed by a workgroup barrier.
+// s_pref[g] = sum of weight(g') over groups g' < g (s_pref[G] = the total, s_pref[G + 1] = the largest
+// weight); computed by the first wave, followed by a workgroup barrier.
 template <class E, class W>
 __device__ __forceinline__ void scan_groups(const GemmArgs& p, int* s_pref, int tid, int lane, E end_of, W weight) {
   if (tid < 64) {
@@ -199,7 +199,7 @@ __device__ __forceinline__ void scan_groups(const GemmArgs& p, int* s_pref, int 
     // LDS, then the lanes' totals are scanned and added to each lane's own entries.
     const int per = (p.G + 63) / 64;
     const int g0 = tid * per;
-    int sum = 0;
+    int sum = 0, mx = 0;
     if (per <= 4) {
       // up to 256 groups: the lane's five group ends are requested together (one memory latency)
       const int last = p.G - 1;
@@ -215,7 +215,9 @@ __device__ __forceinline__ void scan_groups(const GemmArgs& p, int* s_pref, int 
       for (int q = 0; q < 4; ++q) {
         const int g = g0 + q;
         if (q < per && g < p.G) {
-          sum += weight(e[q + 1] - e[q]);
+          const int w = weight(e[q + 1] - e[q]);
+          sum += w;
+          mx = w > mx ? w : mx;
           s_pref[g + 1] = sum;
         }
       }
@@ -225,7 +227,9 @@ __device__ __forceinline__ void scan_groups(const GemmArgs& p, int* s_pref, int 
         const int g = g0 + q;
         if (g < p.G) {
           const int cur = end_of(g);
-          sum += weight(cur - prev);
+          const int w = weight(cur - prev);
+          sum += w;
+          mx = w > mx ? w : mx;
           prev = cur;
           s_pref[g + 1] = sum;
         }
@@ -243,6 +247,12 @@ __device__ __forceinline__ void scan_groups(const GemmArgs& p, int* s_pref, int 
       if (g < p.G) s_pref[g + 1] += base;
     }
     if (tid == 0) s_pref[0] = 0;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int y = __shfl_xor(mx, d);
+      mx = y > mx ? y : mx;
+    }
+    if (tid == 0) s_pref[p.G + 1] = mx;  // the largest weight, after the total
   }
   __syncthreads();
 }
@@ -269,7 +279,10 @@ __device__ __forceinline__ void scan_group_costs(const GemmArgs& p, int* s_pref,
 // workgroups per XCD.
 template <int MODE>
 __device__ __forceinline__ int xcd_first_tile(const GemmArgs& p, const int* s_pref, int total_tiles, int x, int round) {
-  if (MODE != GEMM_K_GROUPED) {
+  // Groups of nearly equal cost (largest within a quarter of the mean): the plain cut by count, which
+  // for a group count that is a multiple of eight also keeps whole groups on one XCD.
+  const bool by_count = MODE != GEMM_K_GROUPED || (int64_t)s_pref[p.G + 1] * p.G * 4 <= (int64_t)s_pref[p.G] * 5;
+  if (by_count) {
     const int per_xcd = (total_tiles + 7) / 8;
     const int t = x * per_xcd;
     return t < total_tiles ? t : total_tiles;

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_pipelined_kerne
                 "every wave must issue the same number of loads per stage");
   constexpr int SC_RING = NS;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [NS][STAGE] operand stages | [SC_RING][BM+BN] fp32 scales
-  __shared__ int s_pref[MODE != GEMM_DENSE ? kMaxGroupsGemm + 1 : 1];
+  __shared__ int s_pref[MODE != GEMM_DENSE ? kMaxGroupsGemm + 2 : 2];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
