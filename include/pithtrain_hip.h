@@ -242,6 +242,21 @@ int pt_group_rows(const int64_t* keys, int64_t m, int32_t num_groups, int32_t al
                   int32_t* offs, int32_t* ks, int64_t* reverse, int32_t* src_of, int64_t cap,
                   void* workspace, int64_t workspace_bytes, pt_stream_t stream);
 
+/* pt_group_rows for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same arguments, results and errors, but
+ * the workspace is a device array built into the library (one copy per GPU, held until the
+ * process ends) instead of an argument, and the call allocates and frees nothing.  It refuses
+ * problems whose pt_group_rows_workspace_bytes(m, num_groups) exceeds
+ * PT_GROUP_ROWS_STATIC_MAX_WORKSPACE (e.g. up to 262144 keys in 256 groups, or 524288 keys in 128).
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two
+ * threads) race; calls on one stream are ordered and need nothing cleared in between.
+ * No counterpart in the reference, which allocates its counters with torch on every call
+ * (token_scatter.py:205-207). */
+#define PT_GROUP_ROWS_STATIC_MAX_WORKSPACE ((1 << 20) + 8192)
+int pt_group_rows_static(const int64_t* keys, int64_t m, int32_t num_groups, int32_t alignment,
+                         int32_t* offs, int32_t* ks, int64_t* reverse, int32_t* src_of, int64_t cap,
+                         pt_stream_t stream);
+
 /* out[r,:] = src_of[r] >= 0 ? in[pre ? pre[src_of[r]] : src_of[r], :] : 0   for r < rows_out,
  * where rows_out = min(cap, round_up(offs_last[0], tail_alignment)) read on the device when
  * offs_last != NULL, else cap.  Rows in [rows_out, cap) are not touched.  elem_bytes-wide

@@ -10,6 +10,7 @@
 // Row movement is a separate pass over the *destination* rows (one wavefront per row, 16-byte
 // accesses) so that padding rows are zeroed and data rows copied in one coalesced sweep.
 #include "common.h"
+#include <mutex>
 
 namespace pt {
 
@@ -589,15 +590,10 @@ extern "C" int64_t pt_group_rows_workspace_bytes(int64_t m, int32_t num_groups) 
   return align_up(W * num_groups * 4, 256) + align_up((int64_t)num_groups * 4, 256);
 }
 
-extern "C" int pt_group_rows(const int64_t* keys, int64_t m, int32_t G, int32_t alignment, int32_t* offs, int32_t* ks,
-                             int64_t* reverse, int32_t* src_of, int64_t cap, void* workspace, int64_t workspace_bytes,
-                             pt_stream_t stream) {
-  PT_REQUIRE(m > 0 && G > 0 && G <= kMaxGroups && alignment > 0, "group_rows: m=%lld G=%d (max %d)", (long long)m, G, kMaxGroups);
-  PT_REQUIRE(m + (int64_t)G * (alignment - 1) < (1ll << 31), "group_rows: row count exceeds int32");
-  PT_REQUIRE(keys && offs && ks && reverse && src_of && workspace, "group_rows: null pointer");
-  PT_REQUIRE(workspace_bytes >= pt_group_rows_workspace_bytes(m, G), "group_rows: workspace too small");
-  PT_REQUIRE(cap >= m, "group_rows: cap < m");
-  hipStream_t s = (hipStream_t)stream;
+// The five launches of the stable counting sort; `workspace` holds the [W][G] chunk counts and the
+// G group starts (pt_group_rows_workspace_bytes), every byte of which is written before it is read.
+static int group_rows_launch(const int64_t* keys, int64_t m, int32_t G, int32_t alignment, int32_t* offs, int32_t* ks,
+                             int64_t* reverse, int32_t* src_of, int64_t cap, void* workspace, hipStream_t s) {
   const int64_t W = cdiv(m, kWaveKeys);
   int32_t* counts = (int32_t*)workspace;
   int32_t* group_start = (int32_t*)((char*)workspace + align_up(W * G * 4, 256));
@@ -609,6 +605,67 @@ extern "C" int pt_group_rows(const int64_t* keys, int64_t m, int32_t G, int32_t 
   gr_scan_groups_kernel<<<1, 1024, 0, s>>>(G, alignment, offs, ks, group_start);
   gr_rank_kernel<<<blocks, 256, lds, s>>>(keys, m, G, bits_for(G), counts, group_start, reverse, src_of, cap);
   return check_launch("group_rows");
+}
+
+static int group_rows_check(const int64_t* keys, int64_t m, int32_t G, int32_t alignment, const int32_t* offs, const int32_t* ks,
+                            const int64_t* reverse, const int32_t* src_of, int64_t cap) {
+  PT_REQUIRE(m > 0 && G > 0 && G <= kMaxGroups && alignment > 0, "group_rows: m=%lld G=%d (max %d)", (long long)m, G, kMaxGroups);
+  PT_REQUIRE(m + (int64_t)G * (alignment - 1) < (1ll << 31), "group_rows: row count exceeds int32");
+  PT_REQUIRE(keys && offs && ks && reverse && src_of, "group_rows: null pointer");
+  PT_REQUIRE(cap >= m, "group_rows: cap < m");
+  return PT_OK;
+}
+
+extern "C" int pt_group_rows(const int64_t* keys, int64_t m, int32_t G, int32_t alignment, int32_t* offs, int32_t* ks,
+                             int64_t* reverse, int32_t* src_of, int64_t cap, void* workspace, int64_t workspace_bytes,
+                             pt_stream_t stream) {
+  if (int rc = group_rows_check(keys, m, G, alignment, offs, ks, reverse, src_of, cap)) return rc;
+  PT_REQUIRE(workspace, "group_rows: null pointer");
+  PT_REQUIRE(workspace_bytes >= pt_group_rows_workspace_bytes(m, G), "group_rows: workspace too small");
+  return group_rows_launch(keys, m, G, alignment, offs, ks, reverse, src_of, cap, workspace, (hipStream_t)stream);
+}
+
+// ---- the same sort for callers that cannot allocate: its workspace is a device array that is
+// part of the loaded code object (one copy per GPU, held until the process ends).  The array's
+// name is only a host-side handle; the address the kernels get is looked up once per device. ----
+static constexpr int64_t kStaticScratchBytes = PT_GROUP_ROWS_STATIC_MAX_WORKSPACE;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on device d, null until looked up
+
+static int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("group_rows_static: no current device (%s)", e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+    return PT_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      set_error("group_rows_static: cannot find the scratch array on device %d: %s", dev, hipGetErrorString(e));
+      return PT_ERR_LAUNCH;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return PT_OK;
+}
+
+extern "C" int pt_group_rows_static(const int64_t* keys, int64_t m, int32_t G, int32_t alignment, int32_t* offs, int32_t* ks,
+                                    int64_t* reverse, int32_t* src_of, int64_t cap, pt_stream_t stream) {
+  if (int rc = group_rows_check(keys, m, G, alignment, offs, ks, reverse, src_of, cap)) return rc;
+  const int64_t need = pt_group_rows_workspace_bytes(m, G);
+  PT_REQUIRE(need <= kStaticScratchBytes,
+             "group_rows_static: m=%lld keys in %d groups need %lld bytes of scratch, the built-in array holds %lld "
+             "(use pt_group_rows with a workspace)",
+             (long long)m, G, (long long)need, (long long)kStaticScratchBytes);
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  return group_rows_launch(keys, m, G, alignment, offs, ks, reverse, src_of, cap, ws, (hipStream_t)stream);
 }
 
 extern "C" int pt_permute_rows(const void* in, int64_t ld_in, void* out, int64_t ld_out, const int32_t* src_of,
