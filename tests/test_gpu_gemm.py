@@ -91,6 +91,40 @@ def test_dense_nt_with_the_reduction_split_over_workgroups(M, N, K):
         _check(partial.double().sum(0), ref, "slabs")
 
 
+def _dense_rows_against_oracle(M, N, K, rows, what):
+    from pith_train_amd.operators.linear import _fp8_gemm_nt
+
+    x, w = _rand((M, K), M + K + 4), _rand((N, K), N + K + 5, 0.02)
+    a, sa, _, _ = Q.fp8cast_rowwise_transpose(x)
+    b, sb, _, _ = Q.fp8cast_blockwise_transpose(w)
+    out = _fp8_gemm_nt(a.cuda(), sa.cuda(), b.cuda(), sb.cuda(), M, N, "cuda", torch.bfloat16)
+    assert out.shape == (M, N)
+    ref = G.gemm_nt_dense(a[rows], sa[rows], b, sb, torch.float64)
+    _check(out[rows.cuda()], ref, what)
+
+
+def test_dense_nt_with_more_tiles_per_workgroup_than_the_tile_table_holds(gemm_kernel):
+    """32768 x 25600 is 12800 tiles of 256 x 256, 50 per workgroup of the persistent kernels: the
+    last tiles of every workgroup are decoded on the fly instead of read from the table built at
+    kernel start.  Two rows of every 256-row tile are compared over all columns, so every tile of
+    the launch is checked."""
+    M, N, K = 32768, 25600, 128
+    rows = torch.arange(0, M, 256).repeat_interleave(2) + torch.tensor([5, 201]).repeat(M // 256)
+    _dense_rows_against_oracle(M, N, K, rows, f"dense {M}x{N}x{K}, {gemm_kernel}")
+
+
+def test_dense_nt_with_an_output_beyond_the_32_bit_store_offsets(gemm_kernel):
+    """A 65536 x 32896 bf16 result is 4.3 GB: past the unsigned 32-bit byte offsets the persistent
+    kernels store through, so the library must route the call to its kernel with 64-bit addresses
+    whatever kernel was asked for.  One row of every 128-row tile, all columns."""
+    if gemm_kernel not in ("auto", "q0"):
+        pytest.skip("the route does not depend on the requested kernel; run twice")
+    M, N, K = 65536, 32896, 128
+    assert M * N * 2 >= 1 << 32
+    rows = torch.arange(0, M, 128) + (torch.arange(M // 128) * 37) % 128
+    _dense_rows_against_oracle(M, N, K, rows, f"dense {M}x{N}x{K} (64-bit route)")
+
+
 def test_dense_scale_extremes():
     """Rows with very different magnitudes: the E8M0 exponents given to the MFMA must be per row."""
     from pith_train_amd.operators.linear import _fp8_gemm_nt
@@ -125,7 +159,12 @@ GROUPED = [
 ]
 
 
-@pytest.mark.parametrize("sizes,N,K", GROUPED)
+# More than 256 groups: the kernels' group scan gives every lane more than four groups (its long
+# path), and the list of tiles is full of empty and single-block groups.
+MANY_GROUPS = [([0 if i % 7 == 3 else (256 if i % 5 == 0 else 128) for i in range(320)], 256, 256)]
+
+
+@pytest.mark.parametrize("sizes,N,K", GROUPED + MANY_GROUPS)
 def test_m_grouped_nt(sizes, N, K):
     from pith_train_amd.operators.grouped_linear import m_grouped_fp8_gemm_nt
 
@@ -180,6 +219,54 @@ def test_m_grouped_nt_scattered_rows(sizes, N, K, gemm_kernel):
     assert (out[untouched] == 7.0).all()
 
 
+def test_m_grouped_nt_with_more_tiles_per_workgroup_than_the_tile_table_holds(gemm_kernel):
+    """Four groups of 25600 rows x 8192 columns: 12800 tiles, 50 per workgroup, so the grouped
+    tile decode (group search, row tile inside the group) also runs on the fly for the last tiles.
+    Two rows of every 256-row tile against the oracle, all columns."""
+    from pith_train_amd.operators.grouped_linear import m_grouped_fp8_gemm_nt
+
+    sizes, N, K = [25600] * 4, 8192, 128
+    ks, offs = _groups(sizes)
+    M, Gn = int(offs[-1]), len(sizes)
+    x, w = _rand((M, K), M + K + 6), _rand((Gn, N, K), N + K + 7, 0.02)
+    a, sa, _, _ = Q.fp8cast_rowwise_colwise(x)
+    b, sb, _, _ = Q.fp8cast_blockwise_transpose_batched(w)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    m_grouped_fp8_gemm_nt((a.cuda(), sa.cuda()), (b.cuda(), sb.cuda()), out, offs.cuda())
+    rows = torch.arange(0, M, 256).repeat_interleave(2) + torch.tensor([9, 250]).repeat(M // 256)
+    grp = rows // 25600
+    for g in range(Gn):
+        r = rows[grp == g]
+        ref = G.gemm_nt_dense(a[r], sa[r], b[g], sb[g], torch.float64)
+        _check(out[r.cuda()], ref, f"m-grouped group {g} of {sizes} N={N} K={K}, {gemm_kernel}")
+
+
+def test_k_grouped_wgrad_with_more_tiles_per_workgroup_than_the_tile_table_holds(gemm_kernel):
+    """200 groups of one 128-row block, 2048 x 2048 results: 12800 tiles, 50 per workgroup.  Groups
+    spread over the whole list (the on-the-fly decode handles the end of every XCD's share) are
+    compared with the oracle; all others must at least be finite and non-trivial."""
+    from pith_train_amd.operators.grouped_linear import k_grouped_fp8_wgrad
+
+    if gemm_kernel == "t":
+        pytest.skip("the tile-per-workgroup kernel has no tile table")
+    Gn, N, K = 200, 2048, 2048
+    ks, offs = _groups([128] * Gn)
+    M = int(offs[-1])
+    dy, x = _rand((M, N), M + N + 1), _rand((M, K), M + K + 2)
+    _, _, dy_ch, dy_s = Q.fp8cast_rowwise_colwise(dy)
+    _, _, x_ch, x_s = Q.fp8cast_rowwise_colwise(x)
+    tr = lambda q: q.view(torch.uint8).T.contiguous().view(torch.float8_e4m3fn).cuda()  # noqa: E731
+    out = torch.full((Gn, N, K), float("nan"), dtype=torch.bfloat16, device="cuda")
+    k_grouped_fp8_wgrad((tr(dy_ch), dy_s.cuda()), (tr(x_ch), x_s.cuda()), out, offs.cuda(), False)
+    assert torch.isfinite(out).all()
+    assert (out.float().abs().amax(dim=(1, 2)) > 0).all()
+    for g in list(range(23, Gn, 25)) + [0, Gn - 1]:  # 24, 49, ..., 199: the last group of every eighth of the list
+        sl = slice(g * 128, (g + 1) * 128)
+        ref = G.gemm_k_grouped_wgrad(dy_ch[sl], dy_s[g : g + 1], x_ch[sl], x_s[g : g + 1], torch.tensor([128], dtype=torch.int32), 1,
+                                     torch.float64).double()
+        _check(out[g : g + 1], ref, f"wgrad group {g} of {Gn}, {gemm_kernel}")
+
+
 # Skewed group sizes: the weight-gradient tiles are shared out over the XCDs by cost (a tile's
 # reduction length), so the cuts fall inside groups, at empty groups and at the ends of the list.
 SKEWED = [
@@ -190,7 +277,7 @@ SKEWED = [
 ]
 
 
-@pytest.mark.parametrize("sizes,N,K", GROUPED + SKEWED)
+@pytest.mark.parametrize("sizes,N,K", GROUPED + SKEWED + MANY_GROUPS)
 @pytest.mark.parametrize("accumulate", [False, True])
 def test_k_grouped_wgrad(sizes, N, K, accumulate):
     from pith_train_amd.operators.grouped_linear import k_grouped_fp8_wgrad
@@ -253,21 +340,3 @@ def test_k_grouped_wgrad_on_column_slices_of_the_scale_array():
         out = torch.full((Gn, half, K), float("nan"), dtype=torch.bfloat16, device="cuda")
         k_grouped_fp8_wgrad((dy_t[lo : lo + half], dy_sc[:, lo : lo + half]), (x_t, x_sc), out, offs.cuda(), False)
         _check(out, ref, f"wgrad on scale columns {lo}..{lo + half}")
-
-
-def test_mfma_rate_probe_runs_and_counts_its_work():
-    """The measurement aid bench.py times: launches, fills its sink, reports 2 * 32 * 32 * 64 FLOP
-    per instruction x 8 per iteration x 4 waves per workgroup."""
-    import ctypes
-
-    from pith_train_amd import _lib
-
-    blocks, iters = 64, 10
-    sink = torch.full((blocks * 256,), float("nan"), device="cuda")
-    flop = ctypes.c_double()
-    _lib.call("pt_probe_mfma_rate", blocks, iters, sink.data_ptr(), ctypes.addressof(flop), _lib.stream_ptr(sink.device))
-    torch.cuda.synchronize()
-    assert flop.value == 2.0 * 32 * 32 * 64 * 8 * iters * 4 * blocks
-    assert torch.isfinite(sink).all() and (sink > 0).all()
-    with pytest.raises(_lib.PithTrainHipError):
-        _lib.call("pt_probe_mfma_rate", 0, iters, sink.data_ptr(), ctypes.addressof(flop), _lib.stream_ptr(sink.device))
