@@ -298,14 +298,27 @@ static bool prefer_pipelined(const GemmArgs& g) {
   }
 }
 
+// The persistent kernels address operands through 32-bit buffer offsets (signed range for the
+// loads, whose out-of-range marker is bit 31) and the result through an unsigned 32-bit byte
+// offset from the start of the output (of one group's block in the k-grouped mode, of the
+// scattered output when rows are stored through an index).  Larger problems go to the
+// tile-per-workgroup kernel, which uses 64-bit pointers.
+static bool fits_persistent(const GemmArgs& g) {
+  const int64_t lim = (1ll << 31) - 1;
+  const int64_t esz = g.out_dtype == PT_F32 ? 4 : 2;
+  const int64_t out_rows = g.out_row_index ? g.out_rows : g.rows_a;
+  const int64_t out_extent = out_rows * g.ldo * esz;
+  return g.a_bytes < lim && g.b_bytes < lim && g.sa_bytes < lim && g.sb_bytes < lim && g.rows_a < lim && g.rows_b < lim &&
+         g.red < lim && out_extent < (1ll << 32);
+}
+
 static int dispatch_gemm(const GemmArgs& g, hipStream_t stream) {
   const int impl = gemm_impl();
-  // the persistent kernels address operands through 32-bit buffer offsets
-  const int64_t lim = (1ll << 31) - 1;
-  const bool fits = g.a_bytes < lim && g.b_bytes < lim && g.sa_bytes < lim && g.sb_bytes < lim && g.rows_a < lim &&
-                    g.rows_b < lim && g.red < lim;
+  const bool fits = fits_persistent(g);
   PT_REQUIRE((!g.out_row_index && !g.bias) || (impl != IMPL_TILE && fits),
-             "gemm: scattered output rows and the fused bias need the persistent kernels");
+             "gemm: scattered output rows and the fused bias need the persistent kernels, which address every operand and "
+             "the output (one group's block of it in the k-grouped mode) through 32-bit byte offsets: operands below 2 GiB, "
+             "output below 4 GiB");
   if (impl == IMPL_TILE || !fits) return launch_gemm<128, 128, 2, 2>(g, stream);
   if (impl == IMPL_AUTO) return prefer_pipelined(g) ? launch_gemm_pipelined(g, 0, stream) : launch_gemm_persistent(g, 0, stream);
   if (impl >= IMPL_PIPELINED) return launch_gemm_pipelined(g, impl - IMPL_PIPELINED, stream);

@@ -57,6 +57,27 @@ def test_gemm_kernel_selection_validates_names_without_a_gpu():
     assert lib.pt_gemm_select_kernel(None) == 0
 
 
+def test_fused_gemm_stores_refuse_outputs_beyond_the_32_bit_store_offsets():
+    """The persistent GEMM kernels address the output through an unsigned 32-bit byte offset.  A
+    biased or scattered store has no 64-bit fallback, so an output of 4 GiB or more is refused on
+    the host, before any launch (the pointers below are never dereferenced)."""
+    from pith_train_amd import _lib
+
+    lib = _lib.load()
+    p = ctypes.c_void_p(0x10000)
+    I64, I32 = ctypes.c_int64, ctypes.c_int32
+    M, N, K, G = 128 * 20000, 1024, 128, 4  # operands 328 MB and 0.5 MB, bf16 output 5.2 GB
+    assert M * N * 2 >= 1 << 32 and M * K < (1 << 31)
+    lib.pt_gemm_m_grouped_nt_bias.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int, ctypes.c_void_p, I32, I64, I64, I64,
+                                              ctypes.c_void_p, ctypes.c_void_p]
+    rc = lib.pt_gemm_m_grouped_nt_bias(p, p, p, p, p, 0, p, G, M, N, K, p, None)
+    assert rc != 0 and b"4 GiB" in lib.pt_last_error()
+    lib.pt_gemm_m_grouped_nt_scatter.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int, ctypes.c_void_p, I32, I64, I64, I64,
+                                                 ctypes.c_void_p, I64, ctypes.c_void_p]
+    rc = lib.pt_gemm_m_grouped_nt_scatter(p, p, p, p, p, 0, p, G, 1024, N, K, p, M, None)
+    assert rc != 0 and b"4 GiB" in lib.pt_last_error()
+
+
 def test_operators_refuse_cpu_tensors_loudly():
     from pith_train_amd import _lib
     from pith_train_amd.operators.deepgemm_quantize import fp8cast_rowwise_colwise
