@@ -400,28 +400,6 @@ def cpu_baseline(kind, H, I, E, k, T, zipf, budget_s=12.0):
     }
 
 
-def mfma_sustained_tflops():
-    """Rate of back-to-back FP8 MFMAs on register operands (library probe), timed with events."""
-    import ctypes
-
-    import torch
-
-    from pith_train_amd import _lib
-
-    blocks, iters = 1024, 2000
-    sink = torch.empty(blocks * 256, device="cuda")
-    flop = ctypes.c_double()
-    stream = _lib.stream_ptr(sink.device)
-    _lib.call("pt_probe_mfma_rate", blocks, 50, sink.data_ptr(), ctypes.addressof(flop), stream)
-    torch.cuda.synchronize()
-    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    a.record()
-    _lib.call("pt_probe_mfma_rate", blocks, iters, sink.data_ptr(), ctypes.addressof(flop), stream)
-    b.record()
-    torch.cuda.synchronize()
-    return flop.value / (a.elapsed_time(b) * 1e-3) / 1e12
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -554,7 +532,6 @@ def main():
         torch.cuda.synchronize()
         assert torch.equal(csrc, cdst)
 
-    sustained = mfma_sustained_tflops()
     result = {
         "metric": "MoE-layer fwd+bwd TFLOP/s (FP8 grouped-expert path, Qwen3-30B-A3B shape, 1 GPU)"
         if args.workload == "qwen3-30b-a3b-moe" else f"MoE-layer fwd+bwd TFLOP/s ({args.workload})",
@@ -592,10 +569,6 @@ def main():
             # every launch priced at the better of the two peaks: what the step's GEMMs would take on
             # a machine that reaches 5 PFLOP/s and 8 TB/s at once
             "floor_ms_per_step": floor_ms,
-            # what a register-only loop of the same MFMA instruction sustains on this box right now
-            # (the clock held under matrix load is below nominal): context for `frac`, not its peak
-            "mfma_register_loop_tflops": sustained,
-            "frac_of_register_loop": achieved / sustained if sustained else None,
             "frac_of_floor": floor_ms / (gemm_ms / max(args.steps, 1)) if gemm_ms > 0 else 0.0,
         },
         **extra,

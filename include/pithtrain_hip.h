@@ -453,13 +453,6 @@ int pt_cross_entropy_fwd(void* logits, int64_t ld, int dtype, const int64_t* tar
 int pt_cross_entropy_bwd(void* grad, int64_t ld, int dtype, int64_t N, int64_t V,
                          const float* grad_output, pt_stream_t stream);
 
-/* Measurement aid without a counterpart in the reference: `blocks` workgroups of four waves issue
- * `iters` x 8 back-to-back v_mfma_scale_f32_32x32x64_f8f6f4 on register operands (no memory
- * traffic).  sink receives blocks * 256 floats; *flop the work of the launch.  Timed by the
- * benchmark to report the matrix rate the part sustains next to its published peak. */
-int pt_probe_mfma_rate(int32_t blocks, int32_t iters, float* sink, double* flop,
-                       pt_stream_t stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -57,7 +57,6 @@ SIGNATURES = {
     "pt_moe_combine_ep_index": (c_int, [P, I64, I64, P, P]),
     "pt_moe_combine_ep_fwd": (c_int, [P, I64, I64, P, P, P, I64, P, I64, I64, I32, I64, c_int, P]),
     "pt_moe_combine_ep_bwd": (c_int, [P, I64, P, I64, I64, P, P, P, I64, P, I64, I32, I64, c_int, P]),
-    "pt_probe_mfma_rate": (c_int, [I32, I32, P, P, P]),
     "pt_group_rows_workspace_bytes": (I64, [I64, I32]),
     "pt_group_rows": (c_int, [P, I64, I32, I32, P, P, P, P, I64, P, I64, P]),
     "pt_group_rows_static": (c_int, [P, I64, I32, I32, P, P, P, P, I64, P]),

@@ -21,10 +21,6 @@
 #include "gemm_persistent_parts.h"
 #include <type_traits>
 
-#ifndef PT_DMA_SLOTS
-#define PT_DMA_SLOTS 64
-#endif
-
 namespace pt {
 
 template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC>
@@ -291,7 +287,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_pipelined_kerne
       // between them (scheduling barriers pin the order): one wavefront keeps its SIMD's matrix
       // pipe fed while it does its own data movement.
       constexpr int NM = TM * TN, NR = TM + TN, NP = DPW + SPW;
-      constexpr int DMA_SLOTS = PT_DMA_SLOTS < NM ? PT_DMA_SLOTS : NM;
+      constexpr int DMA_SLOTS = NM;  // the direct-to-LDS loads are spread over all MFMA slots of the second half
       auto half_a = [&](auto act) {
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
