@@ -73,18 +73,31 @@ def make_dedup_expand(rows, fraction, seed=0):
     return idx[torch.randperm(rows, generator=g)], U
 
 
+ZIPF_BIAS_SCALE = {}  # zipf_s -> factor the popularity bias was multiplied by (reported in the bench line)
+
+
 def make_routing(T, E, k, seed=0, zipf_s=None):
     """Router logits ~N(0,1) (+ an optional Zipf(s) popularity bias: log-probabilities of a seeded
-    random ranking, centred) -> softmax -> top-k expert ids [T, k]."""
+    random ranking, centred) -> softmax -> top-k expert ids [T, k].  The skewed workload asks for
+    routing with at least one empty expert and one above four times the mean count: the bias is
+    multiplied by 1.25, 1.5, ... until the counts say so, and the factor is reported."""
     import torch
 
     g = torch.Generator().manual_seed(seed)
     logits = torch.randn((T, E), generator=g)
-    if zipf_s is not None:
-        ranks = torch.randperm(E, generator=g).float() + 1.0
-        logp = -zipf_s * ranks.log()
-        logits = logits + (logp - logp.mean())
-    return torch.topk(logits.softmax(dim=-1), k=k, dim=-1).indices
+    if zipf_s is None:
+        return torch.topk(logits.softmax(dim=-1), k=k, dim=-1).indices
+    ranks = torch.randperm(E, generator=g).float() + 1.0
+    logp = -zipf_s * ranks.log()
+    bias, scale = logp - logp.mean(), 1.0
+    while True:
+        idx = torch.topk((logits + scale * bias).softmax(dim=-1), k=k, dim=-1).indices
+        counts = torch.bincount(idx.reshape(-1), minlength=E)
+        if ((counts == 0).any() and counts.max() > 4 * counts.float().mean()) or scale >= 8.0:
+            break
+        scale += 0.25
+    ZIPF_BIAS_SCALE[zipf_s] = scale
+    return idx
 
 
 def gemm_flops(rows, H, I):
@@ -548,7 +561,11 @@ def main():
         "data": "synthetic (seed 0: x~N(0,1) bf16, weights~N(0,0.02), grad~N(0,1), router logits~N(0,1) softmax top-k)",
         "config": {
             "workload": args.workload, "kind": kind, "hidden": H, "moe_intermediate": I, "experts": E,
-            "top_k": k, "tokens": T, "routed_rows": rows, "zipf_s": zipf, **extras,
+            "top_k": k, "tokens": T, "routed_rows": rows, "zipf_s": zipf,
+            **({"zipf_bias": "b_e = scale * (log p_e - mean(log p)), p_e ~ rank_e^-s, ranks from a seeded permutation; "
+                             "scale raised in steps of 0.25 until an expert is empty and one exceeds 4x the mean",
+                "zipf_bias_scale": ZIPF_BIAS_SCALE.get(zipf)} if zipf is not None else {}),
+            **extras,
             "algorithmic_gemm_tflop_per_step": flops / 1e12,
             "weight_quant_in_step": True,
         },

@@ -116,14 +116,28 @@ def gemm_flops(m_rows: int, hidden: int, inter: int, fwd_bwd: bool = True) -> fl
     return fwd * (3 if fwd_bwd else 1)
 
 
-def make_routing(num_tokens: int, num_experts: int, top_k: int, seed: int = 0, zipf_s: float | None = None):
-    """Router logits ~N(0,1) (+ optional Zipf(s) popularity bias) -> softmax -> top-k ids [T,k]."""
+def make_routing(num_tokens: int, num_experts: int, top_k: int, seed: int = 0, zipf_s: float | None = None,
+                 return_scale: bool = False):
+    """Router logits ~N(0,1) (+ optional Zipf(s) popularity bias) -> softmax -> top-k ids [T,k].
+
+    The Zipf bias is ``b_e = log p_e - mean(log p)`` with ``p_e`` proportional to ``rank_e ** -s``
+    (ranks from a seeded permutation).  The skewed configuration asks for routing in which some
+    expert gets no token and another more than four times the mean; when the bias as stated does
+    not produce that, it is multiplied by 1.25, 1.5, ... until it does (``return_scale`` also
+    returns that factor)."""
     g = torch.Generator().manual_seed(seed)
     logits = torch.randn((num_tokens, num_experts), generator=g)
-    if zipf_s is not None:
+    scale = 1.0
+    if zipf_s is None:
+        idx = torch.topk(logits.softmax(dim=-1), k=top_k, dim=-1).indices
+    else:
         ranks = torch.randperm(num_experts, generator=g).float() + 1.0
         logp = -zipf_s * ranks.log()
-        logits = logits + (logp - logp.mean())
-    scores = logits.softmax(dim=-1)
-    _, idx = torch.topk(scores, k=top_k, dim=-1)
-    return idx
+        bias = logp - logp.mean()
+        while True:
+            idx = torch.topk((logits + scale * bias).softmax(dim=-1), k=top_k, dim=-1).indices
+            counts = torch.bincount(idx.reshape(-1), minlength=num_experts)
+            if ((counts == 0).any() and counts.max() > 4 * counts.float().mean()) or scale >= 8.0:
+                break
+            scale += 0.25
+    return (idx, scale) if return_scale else idx

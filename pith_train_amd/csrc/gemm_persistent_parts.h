@@ -308,22 +308,19 @@ __device__ __forceinline__ int xcd_first_tile(const GemmArgs& p, const int* s_pr
 // Geometry of logical tile t; plain per-lane arithmetic (every lane may ask for a different t).
 template <int MODE, int BM, int BN>
 __device__ __forceinline__ void decode_tile(const GemmArgs& p, const int* s_pref, int t, Tile& T) {
-  // The 32 CUs of an XCD work on 32 consecutive logical tiles at a time; laying those out as a
-  // 4 x 8 block of the output makes them share 4 a-tiles and 8 b-tiles in that XCD's L2 instead
-  // of 32 a-tiles and 1 b-tile.
+  // The 32 CUs of an XCD work on 32 consecutive logical tiles at a time.  The b-tiles are cut into
+  // strips of at most 8 (of nearly equal width), and a strip is walked row by row: 32 consecutive
+  // tiles then share 32 / w a-tiles and w b-tiles in that XCD's L2 (4 and 8 for a full strip)
+  // instead of 32 a-tiles and 1 b-tile, whatever the number of b-tiles is.
   auto blocked = [&](int t, int& ta, int& tb) {
-    const int full_a = p.tiles_a & ~3, full_b = p.tiles_b & ~7;
-    const int nblk = (full_a >> 2) * (full_b >> 3);
-    if (t < nblk * 32) {
-      const int blk = t >> 5, in = t & 31;
-      ta = (blk % (full_a >> 2)) * 4 + (in & 3);
-      tb = (blk / (full_a >> 2)) * 8 + (in >> 2);
-    } else {  // ragged fringe: remaining columns of tiles, then remaining rows
-      const int r = t - nblk * 32;
-      const int fringe_b = p.tiles_b - full_b;  // extra b-tiles, all a-tiles
-      if (r < fringe_b * p.tiles_a) { ta = r % p.tiles_a; tb = full_b + r / p.tiles_a; }
-      else { const int r2 = r - fringe_b * p.tiles_a; ta = full_a + r2 % (p.tiles_a - full_a); tb = r2 / (p.tiles_a - full_a); }
-    }
+    const int ns = (p.tiles_b + 7) >> 3;           // strips
+    const int w0 = p.tiles_b / ns, wide = p.tiles_b - w0 * ns;  // the first `wide` strips have w0 + 1 b-tiles
+    const int per_wide = p.tiles_a * (w0 + 1);
+    int s, r, w, b0;
+    if (t < wide * per_wide) { s = t / per_wide; r = t - s * per_wide; w = w0 + 1; b0 = s * w; }
+    else { const int t2 = t - wide * per_wide; s = t2 / (p.tiles_a * w0); r = t2 - s * p.tiles_a * w0; w = w0; b0 = wide * (w0 + 1) + s * w0; }
+    ta = r / w;
+    tb = b0 + r - ta * w;
   };
   if (MODE == GEMM_DENSE) {
     T.g = 0;

@@ -130,3 +130,213 @@ def test_full_size_dense_weight_gradient_split_over_the_reduction_matches_the_si
         ref = G.gemm_nt_dense(gt[rows].cpu(), gt_s[rows].cpu(), xt.cpu(), xt_s.cpu(), torch.float64)
         got = split[rows].cpu().double()
         assert ((got - ref).abs() <= 1e-2 * ref.abs() + 1e-2 * ref.pow(2).mean().sqrt()).all()
+
+
+# ---------------------------------------------------------------------------------------------
+# The other configurations at their full sizes, same pattern: the oracle on a few experts (their
+# rows and weights only), size-independent properties for the rest.
+# ---------------------------------------------------------------------------------------------
+def _layer_inputs(kind, hidden, inter, experts, top_k, tokens, zipf=None, seed=0):
+    ids = OM.make_routing(tokens, experts, top_k, seed=seed, zipf_s=zipf)
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((tokens, hidden), generator=g).bfloat16()
+    dy = torch.randn((tokens * top_k, hidden), generator=g).bfloat16()
+    r = lambda *s: (torch.randn(s, generator=g) * 0.02).bfloat16()  # noqa: E731
+    if kind == "split":
+        w = {"gate_proj": r(experts, inter, hidden), "up_proj": r(experts, inter, hidden), "down_proj": r(experts, hidden, inter)}
+    elif kind == "fused":
+        w = {"gate_up_proj": r(experts, 2 * inter, hidden), "down_proj": r(experts, hidden, inter)}
+    else:
+        w = {"gate_up_proj": r(experts, 2 * inter, hidden), "gate_up_proj_bias": r(experts, 2 * inter),
+             "down_proj": r(experts, hidden, inter), "down_proj_bias": r(experts, hidden)}
+    return x, ids.reshape(-1), dy, w
+
+
+def _build(kind, hidden, inter, experts, w):
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules import experts as X
+
+    cls = {"split": X.DeepSeekV2Experts, "fused": X.Qwen35MoeExperts, "gpt_oss": X.GptOssExperts}[kind]
+    mod = cls(hidden, inter, experts).cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        for n, v in w.items():
+            p = getattr(mod, n)
+            (p if kind == "gpt_oss" else p.weight).copy_(v.cuda())
+    FP8WeightCacheControl.step()
+    return mod
+
+
+def _grads(kind, mod, names):
+    return {n: (getattr(mod, n) if kind == "gpt_oss" else getattr(mod, n).weight).grad for n in names}
+
+
+def _run_layer(kind, dims, tokens, eidx, dy, w, expand_idx=None, **kw):
+    from pith_train_amd.modules import experts as X
+
+    hidden, inter, experts = dims
+    mod = _build(kind, hidden, inter, experts, w)
+    tok = tokens.cuda().requires_grad_(True)
+    out = X.forward_stage3(mod, tok, eidx.cuda(), experts, expand_idx=None if expand_idx is None else expand_idx.cuda(), **kw)
+    out.backward(dy.cuda())
+    return out.detach(), tok.grad, _grads(kind, mod, w)
+
+
+def test_deepseek_v2_lite_layer_at_full_size_with_zipf_routing():
+    """64 experts x 1408, top-6, 8192 tokens, Zipf(1.2) popularity bias: an expert without tokens,
+    one with more than four times the mean, an ordinary one - each against the oracle run on its
+    own rows; the empty expert's weight gradients are exact zeros."""
+    hidden, inter, experts, top_k, tokens = 2048, 1408, 64, 6, 8192
+    x, eidx, dy, w = _layer_inputs("split", hidden, inter, experts, top_k, tokens, zipf=1.2)
+    counts = torch.bincount(eidx, minlength=experts)
+    assert (counts == 0).any() and counts.max() > 4 * counts.float().mean(), "the routing must be skewed as the configuration says"
+    rows_in = x.unsqueeze(1).expand(-1, top_k, -1).reshape(-1, hidden).contiguous()
+    out, gtok, grads = _run_layer("split", (hidden, inter, experts), rows_in, eidx, dy, w)
+    assert out.shape == (tokens * top_k, hidden) and torch.isfinite(out.float()).all() and torch.isfinite(gtok.float()).all()
+    empty = int((counts == 0).nonzero()[0])
+    crowded = int(counts.argmax())
+    ordinary = int((counts - counts.float().mean()).abs().argmin())
+    for n in w:
+        assert not grads[n][empty].any(), f"{n}: an expert without tokens has an exactly zero gradient"
+    for e in (crowded, ordinary):
+        rows = (eidx == e).nonzero().flatten()
+        sub_w = {k: v[e : e + 1] for k, v in w.items()}
+        ref = OM.moe_layer_fwd_bwd(rows_in[rows], torch.zeros_like(rows), sub_w, dy[rows], 1, kind="split", fp8=True,
+                                   accum=torch.float32)
+        _close(out[rows.cuda()], ref["out"], f"expert {e} ({rows.numel()} rows) out")
+        _close(gtok[rows.cuda()], ref["grad_tokens"], f"expert {e} grad_tokens")
+        for n in w:
+            _close(grads[n][e], ref[n][0], f"expert {e} {n} grad")
+    # fused and unfused compositions agree bit for bit on the outputs (the token gradient of the
+    # fused node is one fp32 sum over both projections, the composition adds two bf16 gradients)
+    out_u, _, grads_u = _run_layer("split", (hidden, inter, experts), rows_in, eidx, dy, w, fuse_permute=False)
+    assert torch.equal(out, out_u)
+    for n in w:
+        assert torch.equal(grads[n], grads_u[n]), n
+
+
+def test_deepseek_v2_lite_shared_mlp_forward_and_backward_against_the_fp8_linear_oracle():
+    """The two shared experts as one dense FP8 SwiGLU MLP of width 2816 over all 8192 tokens:
+    forward, token gradient and the three weight gradients against the oracle's FP8 linear
+    (quantise, dequantised float product) composed the same way."""
+    from oracle import epilogue as OE
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules import experts as X
+    from pith_train_amd.modules import training
+
+    hidden, width, tokens = 2048, 2816, 8192
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn((tokens, hidden), generator=g).bfloat16()
+    dy = torch.randn((tokens, hidden), generator=g).bfloat16()
+    w = {n: (torch.randn(s, generator=g) * 0.02).bfloat16()
+         for n, s in (("gate_proj", (width, hidden)), ("up_proj", (width, hidden)), ("down_proj", (hidden, width)))}
+    assert training.fp8, "the FP8 layers are the ones under test"
+    mlp = X.DeepSeekV2MLP(hidden, width).cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        for n, v in w.items():
+            getattr(mlp, n).weight.copy_(v.cuda())
+    FP8WeightCacheControl.step()
+    xin = x.cuda().requires_grad_(True)
+    out = mlp(xin)
+    out.backward(dy.cuda())
+
+    acc = torch.float32
+    gate, sg = G.fp8_linear_forward(x, w["gate_proj"], acc)
+    up, su = G.fp8_linear_forward(x, w["up_proj"], acc)
+    h = OE.silu_mul_fwd(gate, up)
+    ref_out, sd = G.fp8_linear_forward(h, w["down_proj"], acc)
+    dh, ref_down = G.fp8_linear_backward(dy, sd, acc)
+    dgate, dup = OE.silu_mul_bwd(dh, gate, up)
+    dx1, ref_gate = G.fp8_linear_backward(dgate, sg, acc)
+    dx2, ref_up = G.fp8_linear_backward(dup, su, acc)
+    _close(out.detach(), ref_out, "shared MLP out")
+    _close(xin.grad, dx1 + dx2, "shared MLP grad_input")
+    _close(mlp.gate_proj.weight.grad, ref_gate, "shared MLP gate_proj grad")
+    _close(mlp.up_proj.weight.grad, ref_up, "shared MLP up_proj grad")
+    _close(mlp.down_proj.weight.grad, ref_down, "shared MLP down_proj grad")
+
+
+def test_gpt_oss_layer_at_full_size():
+    """32 experts, hidden = intermediate = 2880 (ragged against every 128 / 256 tile), top-4, 16384
+    tokens, biases, clamped SwiGLU on interleaved pairs: two experts against the oracle, the fused
+    node against the operator-by-operator composition."""
+    hidden, inter, experts, top_k, tokens = 2880, 2880, 32, 4, 16384
+    x, eidx, dy, w = _layer_inputs("gpt_oss", hidden, inter, experts, top_k, tokens)
+    rows_in = x.unsqueeze(1).expand(-1, top_k, -1).reshape(-1, hidden).contiguous()
+    out, gtok, grads = _run_layer("gpt_oss", (hidden, inter, experts), rows_in, eidx, dy, w)
+    assert out.shape == (tokens * top_k, hidden) and torch.isfinite(out.float()).all() and torch.isfinite(gtok.float()).all()
+    for e in (0, experts - 1):
+        rows = (eidx == e).nonzero().flatten()
+        sub_w = {k: v[e : e + 1] for k, v in w.items()}
+        ref = OM.moe_layer_fwd_bwd(rows_in[rows], torch.zeros_like(rows), sub_w, dy[rows], 1, kind="gpt_oss", fp8=True,
+                                   accum=torch.float32)
+        _close(out[rows.cuda()], ref["out"], f"expert {e} out")
+        _close(gtok[rows.cuda()], ref["grad_tokens"], f"expert {e} grad_tokens")
+        for n in w:
+            _close(grads[n][e], ref[n][0], f"expert {e} {n} grad")
+
+
+def test_qwen3_layer_at_32768_tokens_with_deduplicated_rows():
+    """262144 routed rows of which a quarter re-use an already received row (``expand_idx``): the
+    one-node path that reads the unique rows through the composed map against (i) the oracle on
+    sampled experts for outputs and weight gradients, (ii) the reference's composition
+    (gather -> scatter -> experts -> gather) bit for bit, gradient of the unique rows included."""
+    hidden, inter, experts, top_k, tokens = 2048, 768, 128, 8, 32768
+    routed = tokens * top_k
+    x, eidx, dy, w = _layer_inputs("fused", hidden, inter, experts, top_k, tokens)
+    g = torch.Generator().manual_seed(1)
+    unique = int(round(routed * 0.75))
+    expand_idx = torch.cat([torch.arange(unique), torch.randint(0, unique, (routed - unique,), generator=g)])
+    expand_idx = expand_idx[torch.randperm(routed, generator=g)]
+    src = (torch.randn((unique, hidden), generator=g)).bfloat16()
+    out, gsrc, grads = _run_layer("fused", (hidden, inter, experts), src, eidx, dy, w, expand_idx=expand_idx)
+    assert out.shape == (routed, hidden) and gsrc.shape == (unique, hidden)
+    for e in (5, 100):
+        rows = (eidx == e).nonzero().flatten()
+        sub_w = {k: v[e : e + 1] for k, v in w.items()}
+        ref = OM.moe_layer_fwd_bwd(src[expand_idx[rows]], torch.zeros_like(rows), sub_w, dy[rows], 1, kind="fused", fp8=True,
+                                   accum=torch.float32)
+        _close(out[rows.cuda()], ref["out"], f"expert {e} out")
+        for n in w:
+            _close(grads[n][e], ref[n][0], f"expert {e} {n} grad")
+    out_u, gsrc_u, grads_u = _run_layer("fused", (hidden, inter, experts), src, eidx, dy, w, expand_idx=expand_idx,
+                                        fuse_expand=False, fuse_permute=False)
+    assert torch.equal(out, out_u) and torch.equal(gsrc, gsrc_u)
+    for n in w:
+        assert torch.equal(grads[n], grads_u[n]), n
+    # rows nobody refers to get a zero gradient; a row referred to twice gets the sum of both
+    used = torch.zeros(unique, dtype=torch.bool)
+    used[expand_idx] = True
+    assert not gsrc[(~used).cuda()].any()
+
+
+@pytest.mark.parametrize("n_in,n_out", [(2048, 4096), (2048, 512), (4096, 2048)])
+def test_attention_projections_at_32768_tokens(n_in, n_out):
+    """q (2048 -> 4096), k / v (2048 -> 512) and o (4096 -> 2048) as FP8Linear at 32768 tokens:
+    sampled rows of the output and of the token gradient, and sampled rows of the weight gradient
+    (each a reduction over all tokens), against the oracle's quantise + float64 product."""
+    from oracle import fp8 as Q
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.operators.linear import FP8Linear
+
+    tokens = 32768
+    g = torch.Generator().manual_seed(n_in + n_out)
+    x = torch.randn((tokens, n_in), generator=g).bfloat16()
+    dy = torch.randn((tokens, n_out), generator=g).bfloat16()
+    wt = (torch.randn((n_out, n_in), generator=g) * 0.02).bfloat16()
+    lin = FP8Linear(n_in, n_out, bias=False).cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(wt.cuda())
+    FP8WeightCacheControl.step()
+    xin = x.cuda().requires_grad_(True)
+    out = lin(xin)
+    out.backward(dy.cuda())
+
+    rows = torch.tensor([0, 1, 127, 128, 4095, 16384, 20001, tokens - 1])
+    w_fp8, w_s, w_t_fp8, w_t_s = Q.fp8cast_blockwise_transpose(wt)
+    x_fp8, x_s, x_t_fp8, x_t_s = Q.fp8cast_rowwise_blockwise_transpose(x)
+    g_fp8, g_s, g_t_fp8, g_t_s = Q.fp8cast_rowwise_transpose(dy)
+    _close(out.detach()[rows.cuda()], G.gemm_nt_dense(x_fp8[rows], x_s[rows], w_fp8, w_s, torch.float64), "out rows")
+    _close(xin.grad[rows.cuda()], G.gemm_nt_dense(g_fp8[rows], g_s[rows], w_t_fp8, w_t_s, torch.float64), "grad_input rows")
+    wrows = torch.tensor([0, 127, 128, n_out - 1])
+    _close(lin.weight.grad[wrows.cuda()], G.gemm_nt_dense(g_t_fp8[wrows], g_t_s[wrows], x_t_fp8, x_t_s, torch.float64),
+           "weight grad rows")
