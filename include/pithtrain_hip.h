@@ -31,7 +31,9 @@ int pt_abi_version(void);
 /* ------------------------------------------------------------------------------------------
  * Blockwise FP8 (e4m3fn) quantisation, power-of-two fp32 scales.
  * Replaces pithtrain/operators/deepgemm_quantize.py (six Triton kernels).
- * x is [M,N] with row stride ldx (elements) and unit column stride.
+ * x is [M,N] with row stride ldx (elements) and unit column stride; dtype PT_BF16, PT_F16 or
+ * PT_F32 (the reference's kernels load any float type and convert to fp32,
+ * deepgemm_quantize.py:141-152).
  * ------------------------------------------------------------------------------------------ */
 
 /* layout of the colwise twin written by pt_quant_rowwise_colwise */
@@ -377,7 +379,8 @@ int pt_segment_sum_rows(const void* x, int64_t x_rows, const int32_t* row_index,
 /* out[t,:] = residual[t,:] + S(sum_j float(moe[t*k+j,:]) * topk_weight[t,j]): fp32 products added in
  * the order j = 0..k-1, the sum rounded to the storage type S (dtype), the addition rounded again.
  * moe is [T*k,H], residual and out [T,H] (leading dimensions in elements), topk_weight fp32 [T,k],
- * 1 <= k <= 16. */
+ * 1 <= k <= 16.  residual may be NULL: out is then the rounded sum itself, the weighted sum that
+ * ends the single-device MoE forward (models/qwen3_moe.py:119). */
 int pt_moe_combine_fwd(const void* moe, int64_t ld_moe, const float* topk_weight,
                        const void* residual, int64_t ld_res, void* out, int64_t ld_out, int64_t T,
                        int32_t k, int64_t H, int dtype, pt_stream_t stream);

@@ -137,8 +137,14 @@ __global__ __launch_bounds__(256) void moe_combine_fwd_kernel(CombineArgs p) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[i] = acc[i] + m[i] * wj;
     }
-    const char* rp = p.res + t * p.ld_res + cb;
     char* op = p.out + t * p.ld_out + cb;
+    if (p.res == nullptr) {
+      // no residual: the rounded sum itself (the weighted sum of the single-device MoE forward)
+      if (p.vec) S::store8(op, acc);
+      else for (int i = 0; i < nval; ++i) S::store1(op + i * S::kBytes, acc[i]);
+      continue;
+    }
+    const char* rp = p.res + t * p.ld_res + cb;
     // round the sum to the storage type, then add the residual and round again
     if (p.vec) {
       float r[8], o[8];
@@ -245,14 +251,14 @@ extern "C" int pt_moe_combine_fwd(const void* moe, int64_t ld_moe, const float* 
                                   pt_stream_t stream) {
   PT_REQUIRE(T >= 0 && H >= 0 && k >= 1 && k <= kMaxTopK, "moe_combine_fwd: bad sizes (1 <= k <= %d)", kMaxTopK);
   if (T == 0 || H == 0) return PT_OK;
-  PT_REQUIRE(moe && topk_weight && residual && out, "moe_combine_fwd: null pointer");
-  PT_REQUIRE(ld_moe >= H && ld_res >= H && ld_out >= H && H < (1ll << 31), "moe_combine_fwd: bad leading dimension");
+  PT_REQUIRE(moe && topk_weight && out, "moe_combine_fwd: null pointer");
+  PT_REQUIRE(ld_moe >= H && (!residual || ld_res >= H) && ld_out >= H && H < (1ll << 31), "moe_combine_fwd: bad leading dimension");
   const int eb = dtype == PT_F32 ? 4 : 2;
   CombineArgs a = {};
   a.moe = (const char*)moe; a.res = (const char*)residual; a.out = (char*)out; a.w = topk_weight;
   a.ld_moe = ld_moe * eb; a.ld_res = ld_res * eb; a.ld_out = ld_out * eb;
   a.k = k; a.H = (uint32_t)H; a.chunks = (uint32_t)cdiv(H, 8);
-  a.vec = H % 8 == 0 && al16(moe) && al16(residual) && al16(out) && a.ld_moe % 16 == 0 && a.ld_res % 16 == 0 && a.ld_out % 16 == 0;
+  a.vec = H % 8 == 0 && al16(moe) && al16(residual) && al16(out) && a.ld_moe % 16 == 0 && (!residual || a.ld_res % 16 == 0) && a.ld_out % 16 == 0;
   return launch_combine<false>(a, T, dtype, (hipStream_t)stream);
 }
 

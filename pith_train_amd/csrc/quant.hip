@@ -53,6 +53,19 @@ template <> struct Loader<bf16_tag> {
     return bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(p));
   }
 };
+struct f16_tag {};
+template <> struct Loader<f16_tag> {
+  static constexpr int kBytes = 2;
+  static __device__ __forceinline__ void load8(const void* p, float* v) {
+    const uint4 u = *reinterpret_cast<const uint4*>(p);
+    v[0] = f16_bits_to_f32(u.x & 0xFFFFu); v[1] = f16_bits_to_f32(u.x >> 16); v[2] = f16_bits_to_f32(u.y & 0xFFFFu);
+    v[3] = f16_bits_to_f32(u.y >> 16); v[4] = f16_bits_to_f32(u.z & 0xFFFFu); v[5] = f16_bits_to_f32(u.z >> 16);
+    v[6] = f16_bits_to_f32(u.w & 0xFFFFu); v[7] = f16_bits_to_f32(u.w >> 16);
+  }
+  static __device__ __forceinline__ float load1(const void* p) {
+    return f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(p));
+  }
+};
 template <> struct Loader<float> {
   static constexpr int kBytes = 4;
   static __device__ __forceinline__ void load8(const void* p, float* v) {
@@ -83,6 +96,31 @@ template <> struct Frag<bf16_tag> {
   __device__ __forceinline__ float get(int i, int j) const { return (j & 1) ? bf16_hi(w[i][j >> 1]) : bf16_lo(w[i][j >> 1]); }
   // Compiler fence on the packed registers: values unpacked before it cannot be kept live
   // across it, so each phase of the kernel unpacks again instead of holding 64 floats.
+  __device__ __forceinline__ void fence() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) fence_row(i);
+  }
+  __device__ __forceinline__ void fence_row(int i) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) asm volatile("" : "+v"(w[i][k]));
+  }
+};
+// fp16 sources (the reference's quantisers take any float type): packed like bf16, unpacked with
+// the half-to-float conversion; none of the packed-bf16 shortcuts apply.
+template <> struct Frag<f16_tag> {
+  uint32_t w[8][4];
+  __device__ __forceinline__ void load_row(int i, const void* p) {
+    const uint4 u = *reinterpret_cast<const uint4*>(p);
+    w[i][0] = u.x; w[i][1] = u.y; w[i][2] = u.z; w[i][3] = u.w;
+  }
+  __device__ __forceinline__ void zero_row(int i) { w[i][0] = w[i][1] = w[i][2] = w[i][3] = 0u; }
+  __device__ __forceinline__ void set(int i, int j, const void* p) {
+    const uint32_t b = *reinterpret_cast<const uint16_t*>(p);
+    w[i][j >> 1] = (j & 1) ? ((w[i][j >> 1] & 0x0000FFFFu) | (b << 16)) : ((w[i][j >> 1] & 0xFFFF0000u) | b);
+  }
+  __device__ __forceinline__ float get(int i, int j) const {
+    return f16_bits_to_f32((j & 1) ? (w[i][j >> 1] >> 16) : (w[i][j >> 1] & 0xFFFFu));
+  }
   __device__ __forceinline__ void fence() {
 #pragma unroll
     for (int i = 0; i < 8; ++i) fence_row(i);
@@ -618,8 +656,10 @@ static int launch_quant(const QuantArgs& a, int dtype, int64_t G, hipStream_t st
     hipLaunchKernelGGL((quant_tile_kernel<bf16_tag, AM, BMODE, BL, BS>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
   else if (dtype == PT_F32)
     hipLaunchKernelGGL((quant_tile_kernel<float, AM, BMODE, BL, BS>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else if (dtype == PT_F16)
+    hipLaunchKernelGGL((quant_tile_kernel<f16_tag, AM, BMODE, BL, BS>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
   else
-    PT_REQUIRE(false, "quant: unsupported dtype %d (bf16 and fp32 only)", dtype);
+    PT_REQUIRE(false, "quant: unsupported dtype %d (bf16, fp16 and fp32 only)", dtype);
   return check_launch("quant_tile_kernel");
 }
 

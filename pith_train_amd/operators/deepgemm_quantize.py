@@ -28,8 +28,8 @@ FP8 = torch.float8_e4m3fn
 
 def _prep2d(x: torch.Tensor) -> torch.Tensor:
     _lib.require_cuda(x)
-    if x.dtype not in (torch.bfloat16, torch.float32):
-        raise TypeError(f"fp8cast: expected bfloat16 or float32 input, got {x.dtype}")
+    if x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise TypeError(f"fp8cast: expected bfloat16, float16 or float32 input, got {x.dtype}")
     if x.shape[-1] > 0 and x.stride(-1) != 1:
         x = x.contiguous()
     return x

@@ -8,7 +8,6 @@ three GEMMs are "1x128-scaled rows times 128x128-scaled rows, NT".
 
 from __future__ import annotations
 
-from typing import Tuple
 
 import torch
 import torch.nn as nn
@@ -100,66 +99,62 @@ def fp8_dgrad_wgrad(grad_2d, weight_t_fp8, scale_weight_t, input_t_fp8, scale_in
     return grad_input, weight_grad
 
 
-@torch.library.custom_op("pith_train_amd::fp8_linear_fwd", mutates_args=())
-def _fp8_linear_fwd(
-    input_2d: torch.Tensor,
-    weight: torch.Tensor,
-    weight_fp8: torch.Tensor,
-    scale_weight: torch.Tensor,
-    weight_t_fp8: torch.Tensor,
-    scale_weight_t: torch.Tensor,
-) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    return fp8_act_weight_gemm(input_2d.contiguous(), weight_fp8, scale_weight)
+def _define_ops(namespace: str):
+    """Registers ``<namespace>::fp8_linear_fwd`` and ``<namespace>::fp8_linear_bwd`` with the schema
+    of the reference's ops (operators/linear.py:86-167): eager kernels, shape-only fake kernels for
+    traced regions, and the autograd link from the forward op to the backward op.  Returns the
+    two op objects."""
+    fwd_schema = ("(Tensor input_2d, Tensor weight, Tensor weight_fp8, Tensor scale_weight, Tensor weight_t_fp8, "
+                  "Tensor scale_weight_t) -> (Tensor, Tensor, Tensor)")
+    bwd_schema = ("(Tensor grad_output_2d, Tensor weight_t_fp8, Tensor scale_weight_t, Tensor input_t_fp8, "
+                  "Tensor scale_input_t, int K) -> (Tensor, Tensor)")
+
+    @torch.library.custom_op(f"{namespace}::fp8_linear_fwd", mutates_args=(), schema=fwd_schema)
+    def fwd(input_2d, weight, weight_fp8, scale_weight, weight_t_fp8, scale_weight_t):
+        return fp8_act_weight_gemm(input_2d.contiguous(), weight_fp8, scale_weight)
+
+    @fwd.register_fake
+    def _(input_2d, weight, weight_fp8, scale_weight, weight_t_fp8, scale_weight_t):
+        rows, red = input_2d.shape
+        dev = input_2d.device
+        return (
+            torch.empty((rows, weight.shape[0]), dtype=input_2d.dtype, device=dev),
+            torch.empty((red, rows), dtype=torch.float8_e4m3fn, device=dev),
+            torch.empty((-(-red // 128), -(-rows // 128)), dtype=torch.float32, device=dev),
+        )
+
+    @torch.library.custom_op(f"{namespace}::fp8_linear_bwd", mutates_args=(), schema=bwd_schema)
+    def bwd(grad_output_2d, weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t, K):
+        return fp8_dgrad_wgrad(grad_output_2d.contiguous(), weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t, K)
+
+    @bwd.register_fake
+    def _(grad_output_2d, weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t, K):
+        rows, cols = grad_output_2d.shape
+        like = dict(dtype=grad_output_2d.dtype, device=grad_output_2d.device)
+        return torch.empty((rows, K), **like), torch.empty((cols, K), **like)
+
+    def remember(ctx, inputs, output):
+        # what the backward op reads: the transposed quantised weight and the transposed quantised
+        # activation the forward op handed back
+        ctx.save_for_backward(inputs[4], inputs[5], output[1], output[2])
+        ctx.K = inputs[0].shape[1]
+
+    def backward(ctx, grad_output, _grad_input_t, _grad_scale_t):
+        grad_input, weight_grad = bwd(grad_output, *ctx.saved_tensors, ctx.K)
+        return grad_input, weight_grad, None, None, None, None
+
+    fwd.register_autograd(backward, setup_context=remember)
+    return fwd, bwd
 
 
-@_fp8_linear_fwd.register_fake
-def _(input_2d, weight, weight_fp8, scale_weight, weight_t_fp8, scale_weight_t):
-    (M, K), N = input_2d.shape, weight.shape[0]
-    output = torch.empty((M, N), dtype=input_2d.dtype, device=input_2d.device)
-    input_t_fp8 = torch.empty((K, M), dtype=torch.float8_e4m3fn, device=input_2d.device)
-    size = ((K + 127) // 128, (M + 127) // 128)
-    scale_input_t = torch.empty(size, dtype=torch.float32, device=input_2d.device)
-    return output, input_t_fp8, scale_input_t
-
-
-@torch.library.custom_op("pith_train_amd::fp8_linear_bwd", mutates_args=())
-def _fp8_linear_bwd(
-    grad_output_2d: torch.Tensor,
-    weight_t_fp8: torch.Tensor,
-    scale_weight_t: torch.Tensor,
-    input_t_fp8: torch.Tensor,
-    scale_input_t: torch.Tensor,
-    K: int,
-) -> Tuple[torch.Tensor, torch.Tensor]:
-    return fp8_dgrad_wgrad(
-        grad_output_2d.contiguous(), weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t, K
-    )
-
-
-@_fp8_linear_bwd.register_fake
-def _(grad_output_2d, weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t, K):
-    M, N = grad_output_2d.shape
-    grad_input = torch.empty((M, K), dtype=grad_output_2d.dtype, device=grad_output_2d.device)
-    weight_grad = torch.empty((N, K), dtype=grad_output_2d.dtype, device=grad_output_2d.device)
-    return grad_input, weight_grad
-
-
-def _fp8_linear_setup_context(ctx, inputs, output):
-    input_2d, _, _, _, weight_t_fp8, scale_weight_t = inputs
-    _, input_t_fp8, scale_input_t = output
-    ctx.save_for_backward(weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t)
-    ctx.K = input_2d.shape[1]
-
-
-def _fp8_linear_backward(ctx, grad_output, grad_input_t_fp8, grad_scale_input_t):
-    weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t = ctx.saved_tensors
-    grad_input, weight_grad = _fp8_linear_bwd(
-        grad_output, weight_t_fp8, scale_weight_t, input_t_fp8, scale_input_t, ctx.K
-    )
-    return grad_input, weight_grad, None, None, None, None
-
-
-_fp8_linear_fwd.register_autograd(_fp8_linear_backward, setup_context=_fp8_linear_setup_context)
+_fp8_linear_fwd, _fp8_linear_bwd = _define_ops("pith_train_amd")
+try:
+    # The reference registers the same two ops as pithtrain::fp8_linear_fwd / fp8_linear_bwd; code
+    # that finds them by qualified name (torch.ops.pithtrain.*) gets these kernels.  When the
+    # reference's own module was imported first the names are taken and stay the reference's.
+    _define_ops("pithtrain")
+except RuntimeError:
+    pass
 
 
 class FP8Linear(nn.Linear):

@@ -28,25 +28,29 @@ from .. import _lib
 
 class _MoeCombine(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, moe_outs: torch.Tensor, topk_weight: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
-        _lib.require_cuda(moe_outs, topk_weight, residual)
+    def forward(ctx, moe_outs: torch.Tensor, topk_weight: torch.Tensor, residual: torch.Tensor | None) -> torch.Tensor:
+        _lib.require_cuda(moe_outs, topk_weight)
         assert moe_outs.ndim == 2 and topk_weight.ndim == 2, "moe_outs must be [T*k, H], topk_weight [T, k]"
         T, k = topk_weight.shape
         H = moe_outs.shape[1]
         assert moe_outs.shape[0] == T * k, f"moe_outs has {moe_outs.shape[0]} rows, expected {T * k}"
-        assert residual.numel() == T * H and residual.dtype == moe_outs.dtype, "residual must be [T, H] in moe_outs' dtype"
         assert topk_weight.dtype == torch.float32, "topk_weight must be float32 (softmax scores)"
         moe_outs = moe_outs.contiguous()
-        res2d = residual.reshape(T, H).contiguous()
         w = topk_weight.contiguous()
-        out = torch.empty_like(res2d)
+        res_ptr = 0
+        if residual is not None:
+            _lib.require_cuda(residual)
+            assert residual.numel() == T * H and residual.dtype == moe_outs.dtype, "residual must be [T, H] in moe_outs' dtype"
+            res2d = residual.reshape(T, H).contiguous()
+            res_ptr = res2d.data_ptr()
+        out = torch.empty((T, H), dtype=moe_outs.dtype, device=moe_outs.device)
         _lib.call(
-            "pt_moe_combine_fwd", moe_outs.data_ptr(), H, w.data_ptr(), res2d.data_ptr(), H, out.data_ptr(), H,
+            "pt_moe_combine_fwd", moe_outs.data_ptr(), H, w.data_ptr(), res_ptr, H, out.data_ptr(), H,
             T, k, H, _lib.dtype_code(moe_outs.dtype), _lib.stream_ptr(moe_outs.device),
         )  # fmt: skip
         ctx.save_for_backward(moe_outs, w)
-        ctx.res_shape = residual.shape
-        return out.view(residual.shape)
+        ctx.has_residual = residual is not None
+        return out if residual is None else out.view(residual.shape)
 
     @staticmethod
     def backward(ctx, grad_out: torch.Tensor):
@@ -60,15 +64,17 @@ class _MoeCombine(torch.autograd.Function):
             "pt_moe_combine_bwd", g.data_ptr(), H, moe_outs.data_ptr(), H, w.data_ptr(), d_moe.data_ptr(), H,
             d_w.data_ptr(), T, k, H, _lib.dtype_code(moe_outs.dtype), _lib.stream_ptr(moe_outs.device),
         )  # fmt: skip
-        return d_moe, d_w, grad_out
+        return d_moe, d_w, (grad_out if ctx.has_residual else None)
 
 
-def moe_combine(moe_outs: torch.Tensor, topk_weight: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+def moe_combine(moe_outs: torch.Tensor, topk_weight: torch.Tensor, residual: torch.Tensor | None = None) -> torch.Tensor:
     """``residual + (moe_outs.view(T, k, H) * topk_weight[..., None]).sum(1).to(moe_outs.dtype)``.
 
     ``moe_outs`` is ``[T*k, H]`` (row ``t*k + j`` = expert output of token t's j-th choice),
     ``topk_weight`` float32 ``[T, k]``, ``residual`` any shape with ``T*H`` elements; the result
-    has the residual's shape and ``moe_outs``' dtype."""
+    has the residual's shape and ``moe_outs``' dtype.  Without a residual the result is the
+    rounded weighted sum ``[T, H]`` itself (the last line of the models' ``reference_forward``,
+    models/qwen3_moe.py:119)."""
     return _MoeCombine.apply(moe_outs, topk_weight, residual)
 
 

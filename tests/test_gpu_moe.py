@@ -358,3 +358,89 @@ def test_gpt_oss_block_as_one_node_matches_the_composition(kind, E, H, I, T, k, 
                 torch.testing.assert_close(a.float(), b.float(), rtol=2.0**-7, atol=1e-3 * b.float().abs().max().item())
             else:
                 assert torch.equal(a, b), f"{n} gradient differs"
+
+
+@pytest.mark.parametrize("family", ["qwen3", "deepseek_v2", "gpt_oss", "qwen35"])
+def test_moe_block_reference_forward_against_the_oracle_chain(family):
+    """gate -> one row per (token, choice) -> grouped experts -> top-k weighted sum on one device
+    (``*MoE.reference_forward``).  The oracle chain runs on the gate's own selection (the gate
+    kernels have their own parity tests): scatter, FP8 experts and gather from ``oracle.moe``,
+    the weighted sum from ``oracle.combine``, the shared dense MLP from the oracle's FP8 linear;
+    output and the experts' weight gradients are compared."""
+    from oracle import combine as OC
+    from oracle import epilogue as OE
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules import moe as M
+
+    T, H, I, E, k = 384, 256, 256, 8, 2
+    kind = {"qwen3": "split", "deepseek_v2": "split", "gpt_oss": "gpt_oss", "qwen35": "fused"}[family]
+    w = _weights(kind, E, H, I, seed=21)
+    if family == "qwen3":
+        blk = M.Qwen3MoeMoE(H, I, E, k)
+    elif family == "deepseek_v2":
+        blk = M.DeepSeekV2MoE(H, I, E, k, n_shared_experts=2, routed_scaling_factor=1.5)
+    elif family == "gpt_oss":
+        blk = M.GptOssMoE(H, I, E, k)
+    else:
+        blk = M.Qwen35MoeSparseMoeBlock(H, I, E, k, shared_expert_intermediate_size=384)
+    blk = blk.cuda().to(torch.bfloat16)
+    g = torch.Generator().manual_seed(22)
+    gate = blk.router if family == "gpt_oss" else blk.gate
+    with torch.no_grad():
+        gate.weight.copy_((torch.randn(gate.weight.shape, generator=g) / H**0.5).to(gate.weight.dtype).cuda())
+        for n, v in w.items():
+            p = getattr(blk.experts, n)
+            (p if kind == "gpt_oss" else p.weight).copy_(v.cuda())
+        shared = {}
+        mlp = getattr(blk, "shared_experts", None) or getattr(blk, "shared_expert", None)
+        if mlp is not None:
+            for n in ("gate_proj", "up_proj", "down_proj"):
+                p = getattr(mlp, n).weight
+                shared[n] = (torch.randn(p.shape, generator=g) * 0.02).bfloat16()
+                p.copy_(shared[n].cuda())
+        if family == "qwen35":
+            sg = (torch.randn(blk.shared_expert_gate.weight.shape, generator=g) / H**0.5).bfloat16()
+            blk.shared_expert_gate.weight.copy_(sg.cuda())
+    FP8WeightCacheControl.step()
+    x = torch.randn((T, H), generator=g).bfloat16()
+    dy = torch.randn((T, H), generator=g).bfloat16()
+    xin = x.cuda().requires_grad_(True)
+    y = blk.reference_forward(xin)
+    assert y.shape == (T, H) and y.dtype == torch.bfloat16
+    y.backward(dy.cuda())
+    with torch.no_grad():
+        topk_idx, topk_weight, _ = gate(x.cuda())
+    assert topk_idx.shape == (T, k) and topk_weight.dtype == torch.float32
+
+    eidx = topk_idx.cpu().reshape(-1)
+    rows = x.unsqueeze(1).expand(-1, k, -1).reshape(-1, H).contiguous()
+    fwd = OM.moe_layer_fwd_bwd(rows, eidx, w, None, E, kind=kind, fp8=True, accum=torch.float64)
+    zero = torch.zeros((T, H), dtype=torch.bfloat16)
+    ref = OC.combine_fwd(fwd["out"], topk_weight.cpu(), zero)
+    d_moe, _, _ = OC.combine_bwd(dy, fwd["out"], topk_weight.cpu())
+    if mlp is not None:
+        gt, sg_ = G.fp8_linear_forward(x, shared["gate_proj"], torch.float64)
+        up, su_ = G.fp8_linear_forward(x, shared["up_proj"], torch.float64)
+        sh, _ = G.fp8_linear_forward(OE.silu_mul_fwd(gt, up), shared["down_proj"], torch.float64)
+        if family == "qwen35":
+            sh = (torch.sigmoid((x.float() @ sg.float().T).bfloat16().float()).bfloat16() * sh)
+        ref = ref + sh
+    _close(y, ref, f"{family} reference_forward")
+    bwd = OM.moe_layer_fwd_bwd(rows, eidx, w, d_moe, E, kind=kind, fp8=True, accum=torch.float64)
+    for n in w:
+        p = getattr(blk.experts, n)
+        _close((p if kind == "gpt_oss" else p.weight).grad, bwd[n], f"{family} {n} grad")
+    assert xin.grad is not None and torch.isfinite(xin.grad.float()).all() and gate.weight.grad is not None
+
+
+def test_moe_combine_without_a_residual_is_the_rounded_weighted_sum():
+    from oracle import combine as OC
+    from pith_train_amd.operators.moe_combine import moe_combine
+
+    g = torch.Generator().manual_seed(3)
+    T, k, H = 257, 4, 200
+    moe = torch.randn((T * k, H), generator=g).bfloat16()
+    wgt = torch.rand((T, k), generator=g)
+    got = moe_combine(moe.cuda(), wgt.cuda())
+    want = OC.combine_fwd(moe, wgt, torch.zeros((T, H), dtype=torch.bfloat16))
+    assert torch.equal(got.cpu(), want)

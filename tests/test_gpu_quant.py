@@ -127,6 +127,35 @@ def test_blockwise_transpose_batched(G, N, K):
     assert torch.equal(got[1], got[3].transpose(1, 2))
 
 
+def test_all_six_quantisers_take_fp16_sources():
+    """The reference's kernels take any float input (deepgemm_quantize.py:141-152 loads and
+    converts to fp32); fp16 sources must give the oracle's bytes and scales as bf16 and fp32 do,
+    on full tiles and on ragged edges, subnormal halves included."""
+    D = _ops()
+    g = torch.Generator().manual_seed(16)
+
+    def mk(*shape):
+        x = torch.randn(shape, generator=g) * torch.exp2(torch.randint(-20, 8, shape[:-1] + (1,), generator=g).float())
+        return x.to(torch.float16)
+
+    for M, N in ((256, 384), (128, 200), (384, 7168)):
+        x = mk(M, N)
+        for a, r, w in zip(D.fp8cast_rowwise_colwise(x.cuda()), Q.fp8cast_rowwise_colwise(x), ("tok", "tok_s", "ch", "ch_s")):
+            _eq(a, r, f"rowwise_colwise fp16 {w}")
+    offs = torch.tensor([128, 128, 512], dtype=torch.int32)
+    x = mk(512, 256)
+    for a, r, w in zip(D.fp8cast_rowwise_kmajor(x.cuda(), offs.cuda()), Q.fp8cast_rowwise_kmajor(x, offs), ("tok", "tok_s", "km", "km_s")):
+        _eq(a, r, f"rowwise_kmajor fp16 {w}")
+    for M, N in ((7, 300), (256, 512)):
+        x = mk(M, N)
+        for name in ("fp8cast_rowwise_transpose", "fp8cast_rowwise_blockwise_transpose", "fp8cast_blockwise_transpose"):
+            for a, r, w in zip(getattr(D, name)(x.cuda()), getattr(Q, name)(x), "abcd"):
+                _eq(a, r, f"{name} fp16 {M}x{N} output {w}")
+    w3 = mk(3, 200, 300)
+    for a, r, w in zip(D.fp8cast_blockwise_transpose_batched(w3.cuda()), Q.fp8cast_blockwise_transpose_batched(w3), "abcd"):
+        _eq(a, r, f"blockwise_transpose_batched fp16 output {w}")
+
+
 def test_every_bf16_value_roundtrips_like_the_oracle():
     """All 65280 finite bf16 bit patterns in one tensor (rows sorted by magnitude so scales vary)."""
     D = _ops()
