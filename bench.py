@@ -380,15 +380,16 @@ def hbm_kernel_report(H, I, E, rows, eidx, top_k=8, kind="fused", extras=None):
 
 
 def cpu_baseline(kind, H, I, E, k, T, zipf, budget_s=12.0):
-    """The CPU oracle of the same layer on the same seeded inputs: the BF16 grouped-linear
-    semantics (the reference's pure-PyTorch path), forward + backward, all host cores given to
-    torch.  The whole workload is repeated until about ``budget_s`` seconds have been spent."""
+    """The CPU oracle of the same layer on the same seeded inputs, forward + backward, on the
+    threads torch takes by itself on this host (reported as ``cores``).  Two legs: the BF16
+    grouped-linear semantics (the reference's pure-PyTorch path) on the whole workload, repeated
+    until about ``budget_s`` seconds have been spent - the headline CPU figure -, and the FP8 leg
+    (quantise -> dequantise -> fp32 matmul per group) on the rows of a few experts."""
     import torch
 
     from oracle import moe as OM
 
-    cores = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(cores)
+    cores = torch.get_num_threads()
     ids, x, dy, w = make_inputs(kind, H, I, E, k, T, zipf, seed=0)
     tokens = x.unsqueeze(1).expand(-1, k, -1).reshape(-1, H).contiguous()
     eidx = ids.reshape(-1)
@@ -403,6 +404,14 @@ def cpu_baseline(kind, H, I, E, k, T, zipf, budget_s=12.0):
         if el > budget_s or reps >= 20:
             break
     sec = el / reps
+    # FP8 leg on the experts 0 .. n-1 only (their rows, their weights): the oracle's quantisers and
+    # dequantised products are elementwise tensor code, an order of magnitude slower per FLOP
+    n = max(1, E // 16)
+    sel = (eidx < n).nonzero().flatten()
+    sub_w = {name: v[:n] for name, v in w.items()}
+    t1 = time.perf_counter()
+    OM.moe_layer_fwd_bwd(tokens[sel], eidx[sel], sub_w, dy[sel], n, kind=kind, fp8=True, accum=torch.float32)
+    sec8 = time.perf_counter() - t1
     return {
         "value": flops / sec / 1e12,
         "unit": "TFLOP/s",
@@ -410,6 +419,9 @@ def cpu_baseline(kind, H, I, E, k, T, zipf, budget_s=12.0):
         "kind": "port",
         "sample": f"full workload ({T * k} routed rows, {E} experts), bf16 grouped-linear oracle fwd+bwd on the host, "
                   f"{reps} rep(s), {sec:.2f} s each",
+        "fp8_leg": {"value": OM.gemm_flops(int(sel.numel()), H, I) / sec8 / 1e12, "unit": "TFLOP/s", "cores": cores,
+                    "sample": f"quantise -> dequantise -> fp32 matmul oracle on the {int(sel.numel())} rows of experts 0..{n - 1}, "
+                              f"one pass of {sec8:.2f} s"},
     }
 
 

@@ -237,7 +237,8 @@ int64_t pt_group_rows_workspace_bytes(int64_t m, int32_t num_groups);
  *   offs[G] int32 inclusive cumsum of padded sizes, ks[G] int32 padded sizes
  *   reverse[m] int64: destination row of source row i  (reverse_shuffle_idxs)
  *   src_of[cap] int32: source row of destination row r, -1 for pad rows (r < cap)
- * Canonical order: ascending source row inside a group.
+ * Canonical order: ascending source row inside a group.  Keys are expected in [0,num_groups); a row
+ * whose key is outside belongs to no group: no src_of entry names it and its reverse entry is 0.
  * _compute_group_offsets_kernel + slot assignment of _scatter_for_grouped_gemm_kernel,
  * token_scatter.py:38-101. */
 int pt_group_rows(const int64_t* keys, int64_t m, int32_t num_groups, int32_t alignment,

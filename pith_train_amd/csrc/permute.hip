@@ -137,6 +137,10 @@ __global__ __launch_bounds__(256) void gr_rank_kernel(const int64_t* keys, int64
       const int64_t pos = (int64_t)b + rank;
       reverse[i] = pos;
       if (pos < cap) src_of[pos] = (int32_t)i;
+    } else if (i < m) {
+      // a key outside [0, G) belongs to no group: the row is dropped (no src_of entry names it) and
+      // its reverse entry is a valid row, so that a later gather through it stays in bounds
+      reverse[i] = 0;
     }
   }
 }

@@ -31,13 +31,31 @@ from .deepgemm_quantize import (
 )
 
 
+_GROUPED_MM_USABLE: dict = {}  # (device type, dtype) -> whether torch's grouped_mm runs there
+
+
+def _torch_grouped_mm_usable(a: torch.Tensor) -> bool:
+    """Decided once per device type and dtype with a one-group 16 x 16 product, so that an error
+    on real operands (out of memory, a shape mismatch) is raised instead of being turned into the
+    slow per-group loop."""
+    key = (a.device.type, a.dtype)
+    if key not in _GROUPED_MM_USABLE:
+        ok = hasattr(F, "grouped_mm")
+        if ok:
+            try:
+                t = torch.zeros((16, 16), dtype=a.dtype, device=a.device)
+                F.grouped_mm(t, t.unsqueeze(0), offs=torch.tensor([16], dtype=torch.int32, device=a.device))
+            except (RuntimeError, NotImplementedError):
+                ok = False
+        _GROUPED_MM_USABLE[key] = ok
+    return _GROUPED_MM_USABLE[key]
+
+
 def _grouped_mm(a: torch.Tensor, b: torch.Tensor, offs: torch.Tensor) -> torch.Tensor:
-    """``F.grouped_mm`` where torch provides it, otherwise the per-group loop it stands for."""
-    if hasattr(F, "grouped_mm"):
-        try:
-            return F.grouped_mm(a, b, offs=offs)
-        except (RuntimeError, NotImplementedError):
-            pass
+    """``F.grouped_mm`` where torch provides it for the device, otherwise the per-group loop it
+    stands for (which reads the offsets on the host)."""
+    if _torch_grouped_mm_usable(a):
+        return F.grouped_mm(a, b, offs=offs)
     bounds = [0] + offs.tolist()
     if a.dim() == 2 and b.dim() == 3:  # jagged on rows of a
         out = a.new_zeros((a.shape[0], b.shape[2]))
