@@ -148,7 +148,7 @@ class GemmTimer:
     NAMES = ("pt_gemm_m_grouped_nt", "pt_gemm_m_grouped_nt_scatter", "pt_gemm_m_grouped_nt_bias",
              "pt_gemm_m_grouped_nt_scatter_bias", "pt_gemm_k_grouped_wgrad",
              "pt_gemm_k_grouped_wgrad_ld",
-             "pt_gemm_nt_dense", "pt_gemm_nt_dense_splitk")
+             "pt_gemm_nt_dense", "pt_gemm_nt_dense_splitk", "pt_gemm_nt_dense_ld", "pt_gemm_nt_dense_splitk_ld")
 
     def __init__(self):
         self.records = []
@@ -171,6 +171,7 @@ class GemmTimer:
                 b.record()
                 # rows x columns x reduction as the entry point takes them (the three int64 sizes)
                 sizes = {"pt_gemm_nt_dense": args[6:9], "pt_gemm_nt_dense_splitk": args[7:10],
+                         "pt_gemm_nt_dense_ld": args[8:11], "pt_gemm_nt_dense_splitk_ld": args[9:12],
                          "pt_gemm_k_grouped_wgrad": args[9:12],
                          "pt_gemm_k_grouped_wgrad_ld": args[11:14]}.get(name, args[8:11])
                 timer.records.append((name, a, b, "x".join(str(int(v)) for v in sizes)))

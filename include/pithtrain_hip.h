@@ -110,12 +110,23 @@ int pt_clamped_swiglu_bwd_quant_rowwise_colwise(const void* grad_h, int64_t ld_g
 int pt_quant_rowwise_transpose(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
                                void* tok_fp8, float* tok_scale, void* t_fp8, float* t_scale,
                                pt_stream_t stream);
+/* The same with a row pitch ld_t >= M (bytes) for t_fp8: a reduction over all tokens reads the
+ * transposed operand along rows, and a power-of-two pitch (M = 8192, 32768 tokens) puts those rows
+ * on few memory channels.  No counterpart in the reference (its transposed outputs are packed). */
+int pt_quant_rowwise_transpose_ld(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
+                                  void* tok_fp8, float* tok_scale, void* t_fp8, int64_t ld_t,
+                                  float* t_scale, pt_stream_t stream);
 
 /* rowwise(x) + 128x128 blockwise(x^T): blk_t_fp8[K,M], blk_t_scale[ceil(K/128),ceil(M/128)].
  * fp8cast_rowwise_blockwise_transpose, deepgemm_quantize.py:575-629 */
 int pt_quant_rowwise_blockwise_transpose(const void* x, int dtype, int64_t M, int64_t K,
                                          int64_t ldx, void* tok_fp8, float* tok_scale,
                                          void* blk_t_fp8, float* blk_t_scale, pt_stream_t stream);
+/* The same with a row pitch ld_t >= M (bytes) for blk_t_fp8 (see pt_quant_rowwise_transpose_ld). */
+int pt_quant_rowwise_blockwise_transpose_ld(const void* x, int dtype, int64_t M, int64_t K,
+                                            int64_t ldx, void* tok_fp8, float* tok_scale,
+                                            void* blk_t_fp8, int64_t ld_t, float* blk_t_scale,
+                                            pt_stream_t stream);
 
 /* 128x128 blockwise(x) + blockwise(x^T) for x[G,N,K] (element strides stride_g, stride_row):
  * fp8[G,N,K], scale[G,ceil(N/128),ceil(K/128)], fp8_t[G,K,N], scale_t[G,ceil(K/128),ceil(N/128)].
@@ -148,6 +159,11 @@ int pt_quant_blockwise_transpose_batched_into(const void* x, int dtype, int64_t 
 int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const void* b_fp8,
                      const float* b_scale, void* out, int out_dtype, int64_t M, int64_t N,
                      int64_t K, pt_stream_t stream);
+/* The same for operands with row pitches lda, ldb >= K (bytes, multiples of 16): the padded
+ * transposed operands of pt_quant_rowwise_transpose_ld / pt_quant_rowwise_blockwise_transpose_ld. */
+int pt_gemm_nt_dense_ld(const void* a_fp8, int64_t lda, const float* a_scale, const void* b_fp8,
+                        int64_t ldb, const float* b_scale, void* out, int out_dtype, int64_t M,
+                        int64_t N, int64_t K, pt_stream_t stream);
 /* Split-K form of pt_gemm_nt_dense for outputs with too few 256 x 256 tiles to fill the GPU (the
  * weight gradient of a dense linear, linear.py:61-83: M, N = weight dims, K = tokens): the
  * reduction is cut into `splits` ranges of split_len (a multiple of 128), range s is reduced into
@@ -156,6 +172,10 @@ int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const void* b_fp8,
 int pt_gemm_nt_dense_splitk(const void* a_fp8, const float* a_scale, const void* b_fp8,
                             const float* b_scale, float* partial, int32_t splits, int64_t split_len,
                             int64_t M, int64_t N, int64_t K, pt_stream_t stream);
+int pt_gemm_nt_dense_splitk_ld(const void* a_fp8, int64_t lda, const float* a_scale,
+                               const void* b_fp8, int64_t ldb, const float* b_scale, float* partial,
+                               int32_t splits, int64_t split_len, int64_t M, int64_t N, int64_t K,
+                               pt_stream_t stream);
 int pt_sum_partials(const float* partial, int32_t splits, int64_t n, void* out, int out_dtype,
                     pt_stream_t stream);
 

@@ -34,11 +34,15 @@ SIGNATURES = {
     "pt_clamped_swiglu_bwd_quant_rowwise_colwise": (c_int, [P, I64, P, I64, I64, I64, F, F, P, P, P, P, P, P, P]),
     "pt_quant_rowwise_transpose": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, P]),
     "pt_quant_rowwise_blockwise_transpose": (c_int, [P, c_int, I64, I64, I64, P, P, P, P, P]),
+    "pt_quant_rowwise_transpose_ld": (c_int, [P, c_int, I64, I64, I64, P, P, P, I64, P, P]),
+    "pt_quant_rowwise_blockwise_transpose_ld": (c_int, [P, c_int, I64, I64, I64, P, P, P, I64, P, P]),
     "pt_quant_blockwise_transpose_batched": (c_int, [P, c_int, I64, I64, I64, I64, I64, P, P, P, P, P]),
     "pt_quant_blockwise_transpose_batched_into": (c_int, [P, c_int, I64, I64, I64, I64, I64, P, I64, P, I64, P, I64, I64, P, I64,
                                                           I64, P]),
     "pt_gemm_nt_dense": (c_int, [P, P, P, P, P, c_int, I64, I64, I64, P]),
     "pt_gemm_nt_dense_splitk": (c_int, [P, P, P, P, P, I32, I64, I64, I64, I64, P]),
+    "pt_gemm_nt_dense_ld": (c_int, [P, I64, P, P, I64, P, P, c_int, I64, I64, I64, P]),
+    "pt_gemm_nt_dense_splitk_ld": (c_int, [P, I64, P, P, I64, P, P, I32, I64, I64, I64, I64, P]),
     "pt_sum_partials": (c_int, [P, I32, I64, P, c_int, P]),
     "pt_gemm_m_grouped_nt": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P]),
     "pt_gemm_m_grouped_nt_bias": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, P]),

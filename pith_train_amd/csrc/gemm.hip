@@ -338,36 +338,51 @@ extern "C" int pt_gemm_select_kernel(const char* name) {
 
 static bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
-extern "C" int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale, void* out,
-                                int out_dtype, int64_t M, int64_t N, int64_t K, pt_stream_t stream) {
+static int gemm_nt_dense_impl(const void* a_fp8, int64_t lda, const float* a_scale, const void* b_fp8, int64_t ldb,
+                              const float* b_scale, void* out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                              pt_stream_t stream) {
   PT_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_nt_dense: negative size");
   if (M == 0 || N == 0) return PT_OK;
   PT_REQUIRE(K > 0 && K % 16 == 0, "gemm_nt_dense: K=%lld must be a positive multiple of 16", (long long)K);
+  PT_REQUIRE(lda >= K && ldb >= K && lda % 16 == 0 && ldb % 16 == 0, "gemm_nt_dense: row pitches must be multiples of 16 and at least K");
   PT_REQUIRE(a_fp8 && a_scale && b_fp8 && b_scale && out && al16(a_fp8) && al16(b_fp8), "gemm_nt_dense: null or misaligned pointer");
   PT_REQUIRE(out_dtype == PT_BF16 || out_dtype == PT_F32, "gemm_nt_dense: out_dtype must be bf16 or fp32");
   const int64_t KB = cdiv(K, 128);
   GemmArgs g = {};
-  g.a = (const uint8_t*)a_fp8; g.lda = K; g.b = (const uint8_t*)b_fp8; g.ldb = K;
+  g.a = (const uint8_t*)a_fp8; g.lda = lda; g.b = (const uint8_t*)b_fp8; g.ldb = ldb;
   g.sa = a_scale; g.sa_rs = KB; g.sa_ks = 1; g.sa_shift = 0;
   g.sb = b_scale; g.sb_rs = KB; g.sb_ks = 1; g.sb_shift = 7;
   g.out = out; g.ldo = N; g.out_dtype = out_dtype; g.accumulate = 0;
   g.rows_a = M; g.rows_b = N; g.red = K; g.mode = GEMM_DENSE;
-  g.a_bytes = M * g.lda; g.b_bytes = N * g.ldb; g.sa_bytes = M * KB * 4; g.sb_bytes = cdiv(N, 128) * KB * 4;
+  g.a_bytes = (M - 1) * lda + K; g.b_bytes = (N - 1) * ldb + K; g.sa_bytes = M * KB * 4; g.sb_bytes = cdiv(N, 128) * KB * 4;
   g.tiles_a = (int)cdiv(M, 128); g.tiles_b = (int)cdiv(N, 128);
   g.total_tiles = (int64_t)g.tiles_a * g.tiles_b;
   return dispatch_gemm(g, (hipStream_t)stream);
+}
+
+extern "C" int pt_gemm_nt_dense(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale, void* out,
+                                int out_dtype, int64_t M, int64_t N, int64_t K, pt_stream_t stream) {
+  return gemm_nt_dense_impl(a_fp8, K, a_scale, b_fp8, K, b_scale, out, out_dtype, M, N, K, stream);
+}
+
+extern "C" int pt_gemm_nt_dense_ld(const void* a_fp8, int64_t lda, const float* a_scale, const void* b_fp8, int64_t ldb,
+                                   const float* b_scale, void* out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                   pt_stream_t stream) {
+  return gemm_nt_dense_impl(a_fp8, lda, a_scale, b_fp8, ldb, b_scale, out, out_dtype, M, N, K, stream);
 }
 
 // ---- split-K: a dense GEMM whose output has too few tiles to fill the GPU ------------------------
 // The reduction is cut into `splits` ranges of split_len (a multiple of 128, so every range starts
 // on a scale block); range s is computed like a group of the k-grouped mode into the fp32 slab
 // partial[s] (M x N), and pt_sum_partials adds the slabs in the order of s.
-extern "C" int pt_gemm_nt_dense_splitk(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
-                                       float* partial, int32_t splits, int64_t split_len, int64_t M, int64_t N, int64_t K,
-                                       pt_stream_t stream) {
+static int gemm_nt_dense_splitk_impl(const void* a_fp8, int64_t lda, const float* a_scale, const void* b_fp8, int64_t ldb,
+                                     const float* b_scale, float* partial, int32_t splits, int64_t split_len, int64_t M,
+                                     int64_t N, int64_t K, pt_stream_t stream) {
   PT_REQUIRE(M >= 0 && N >= 0 && K >= 0, "gemm_nt_dense_splitk: negative size");
   if (M == 0 || N == 0) return PT_OK;
   PT_REQUIRE(K > 0 && K % 16 == 0, "gemm_nt_dense_splitk: K=%lld must be a positive multiple of 16", (long long)K);
+  PT_REQUIRE(lda >= K && ldb >= K && lda % 16 == 0 && ldb % 16 == 0,
+             "gemm_nt_dense_splitk: row pitches must be multiples of 16 and at least K");
   PT_REQUIRE(splits >= 1 && split_len > 0 && split_len % 128 == 0 && (int64_t)splits * split_len >= K &&
                  (int64_t)(splits - 1) * split_len < K,
              "gemm_nt_dense_splitk: %d ranges of %lld (a multiple of 128) must cover K=%lld with none empty", splits,
@@ -376,16 +391,28 @@ extern "C" int pt_gemm_nt_dense_splitk(const void* a_fp8, const float* a_scale, 
              "gemm_nt_dense_splitk: null or misaligned pointer");
   const int64_t KB = cdiv(K, 128);
   GemmArgs g = {};
-  g.a = (const uint8_t*)a_fp8; g.lda = K; g.b = (const uint8_t*)b_fp8; g.ldb = K;
+  g.a = (const uint8_t*)a_fp8; g.lda = lda; g.b = (const uint8_t*)b_fp8; g.ldb = ldb;
   g.sa = a_scale; g.sa_rs = KB; g.sa_ks = 1; g.sa_shift = 0;
   g.sb = b_scale; g.sb_rs = KB; g.sb_ks = 1; g.sb_shift = 7;
   g.out = partial; g.ldo = N; g.out_dtype = PT_F32; g.accumulate = 0;
   g.rows_a = M; g.rows_b = N; g.red = K; g.mode = GEMM_K_GROUPED; g.offs = nullptr; g.G = splits; g.split_len = split_len;
   g.out_stride_g = M * N;
-  g.a_bytes = M * g.lda; g.b_bytes = N * g.ldb; g.sa_bytes = M * KB * 4; g.sb_bytes = cdiv(N, 128) * KB * 4;
+  g.a_bytes = (M - 1) * lda + K; g.b_bytes = (N - 1) * ldb + K; g.sa_bytes = M * KB * 4; g.sb_bytes = cdiv(N, 128) * KB * 4;
   g.tiles_a = (int)cdiv(M, 128); g.tiles_b = (int)cdiv(N, 128);
   g.total_tiles = (int64_t)g.tiles_a * g.tiles_b * splits;
   return dispatch_gemm(g, (hipStream_t)stream);
+}
+
+extern "C" int pt_gemm_nt_dense_splitk(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
+                                       float* partial, int32_t splits, int64_t split_len, int64_t M, int64_t N, int64_t K,
+                                       pt_stream_t stream) {
+  return gemm_nt_dense_splitk_impl(a_fp8, K, a_scale, b_fp8, K, b_scale, partial, splits, split_len, M, N, K, stream);
+}
+
+extern "C" int pt_gemm_nt_dense_splitk_ld(const void* a_fp8, int64_t lda, const float* a_scale, const void* b_fp8, int64_t ldb,
+                                          const float* b_scale, float* partial, int32_t splits, int64_t split_len, int64_t M,
+                                          int64_t N, int64_t K, pt_stream_t stream) {
+  return gemm_nt_dense_splitk_impl(a_fp8, lda, a_scale, b_fp8, ldb, b_scale, partial, splits, split_len, M, N, K, stream);
 }
 
 namespace pt {

@@ -724,29 +724,57 @@ static int quant_rowwise_colwise_impl(const void* x, int dtype, int64_t M, int64
   PT_REQUIRE(false, "quant_rowwise_colwise: bad ch_layout %d", ch_layout);
 }
 
-extern "C" int pt_quant_rowwise_transpose(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
-                                          void* tok_fp8, float* tok_scale, void* t_fp8,
-                                          float* t_scale, pt_stream_t stream) {
-  PT_REQUIRE(M >= 0 && N >= 0 && ldx >= N, "quant_rowwise_transpose: bad shape");
+static int quant_rowwise_transpose_impl(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx, void* tok_fp8,
+                                        float* tok_scale, void* t_fp8, int64_t ld_t, float* t_scale, pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && N >= 0 && ldx >= N && ld_t >= M, "quant_rowwise_transpose: bad shape");
   if (M == 0 || N == 0) return PT_OK;
   PT_REQUIRE(x && tok_fp8 && tok_scale && t_fp8 && t_scale, "quant_rowwise_transpose: null pointer");
   QuantArgs a;
   fill_common(a, x, dtype, M, N, ldx);
   a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)t_fp8; a.b_scale = t_scale;
+  a.ld_t = ld_t;
+  a.vec_out_t = a.vec_out_t && ld_t % 16 == 0 && ((uintptr_t)t_fp8) % 16 == 0;
   return launch_quant<A_ROW, B_COL, BL_TRANSPOSED, BS_N_MB>(a, dtype, 1, (hipStream_t)stream);
+}
+
+extern "C" int pt_quant_rowwise_transpose(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
+                                          void* tok_fp8, float* tok_scale, void* t_fp8,
+                                          float* t_scale, pt_stream_t stream) {
+  return quant_rowwise_transpose_impl(x, dtype, M, N, ldx, tok_fp8, tok_scale, t_fp8, M, t_scale, stream);
+}
+
+extern "C" int pt_quant_rowwise_transpose_ld(const void* x, int dtype, int64_t M, int64_t N, int64_t ldx,
+                                             void* tok_fp8, float* tok_scale, void* t_fp8, int64_t ld_t,
+                                             float* t_scale, pt_stream_t stream) {
+  return quant_rowwise_transpose_impl(x, dtype, M, N, ldx, tok_fp8, tok_scale, t_fp8, ld_t, t_scale, stream);
+}
+
+static int quant_rowwise_blockwise_transpose_impl(const void* x, int dtype, int64_t M, int64_t K, int64_t ldx, void* tok_fp8,
+                                                  float* tok_scale, void* blk_t_fp8, int64_t ld_t, float* blk_t_scale,
+                                                  pt_stream_t stream) {
+  PT_REQUIRE(M >= 0 && K >= 0 && ldx >= K && ld_t >= M, "quant_rowwise_blockwise_transpose: bad shape");
+  if (M == 0 || K == 0) return PT_OK;
+  PT_REQUIRE(x && tok_fp8 && tok_scale && blk_t_fp8 && blk_t_scale, "quant_rowwise_blockwise_transpose: null pointer");
+  QuantArgs a;
+  fill_common(a, x, dtype, M, K, ldx);
+  a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)blk_t_fp8; a.b_scale = blk_t_scale;
+  a.ld_t = ld_t;
+  a.vec_out_t = a.vec_out_t && ld_t % 16 == 0 && ((uintptr_t)blk_t_fp8) % 16 == 0;
+  return launch_quant<A_ROW, B_BLOCK, BL_TRANSPOSED, BS_MB_N>(a, dtype, 1, (hipStream_t)stream);
 }
 
 extern "C" int pt_quant_rowwise_blockwise_transpose(const void* x, int dtype, int64_t M, int64_t K,
                                                     int64_t ldx, void* tok_fp8, float* tok_scale,
                                                     void* blk_t_fp8, float* blk_t_scale,
                                                     pt_stream_t stream) {
-  PT_REQUIRE(M >= 0 && K >= 0 && ldx >= K, "quant_rowwise_blockwise_transpose: bad shape");
-  if (M == 0 || K == 0) return PT_OK;
-  PT_REQUIRE(x && tok_fp8 && tok_scale && blk_t_fp8 && blk_t_scale, "quant_rowwise_blockwise_transpose: null pointer");
-  QuantArgs a;
-  fill_common(a, x, dtype, M, K, ldx);
-  a.a_out = (uint8_t*)tok_fp8; a.a_scale = tok_scale; a.b_out = (uint8_t*)blk_t_fp8; a.b_scale = blk_t_scale;
-  return launch_quant<A_ROW, B_BLOCK, BL_TRANSPOSED, BS_MB_N>(a, dtype, 1, (hipStream_t)stream);
+  return quant_rowwise_blockwise_transpose_impl(x, dtype, M, K, ldx, tok_fp8, tok_scale, blk_t_fp8, M, blk_t_scale, stream);
+}
+
+extern "C" int pt_quant_rowwise_blockwise_transpose_ld(const void* x, int dtype, int64_t M, int64_t K,
+                                                       int64_t ldx, void* tok_fp8, float* tok_scale,
+                                                       void* blk_t_fp8, int64_t ld_t, float* blk_t_scale,
+                                                       pt_stream_t stream) {
+  return quant_rowwise_blockwise_transpose_impl(x, dtype, M, K, ldx, tok_fp8, tok_scale, blk_t_fp8, ld_t, blk_t_scale, stream);
 }
 
 static int quant_blockwise_transpose_batched_impl(const void* x, int dtype, int64_t G, int64_t N, int64_t K, int64_t stride_g,

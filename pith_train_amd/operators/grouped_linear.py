@@ -54,7 +54,15 @@ def _torch_grouped_mm_usable(a: torch.Tensor) -> bool:
 def _grouped_mm(a: torch.Tensor, b: torch.Tensor, offs: torch.Tensor) -> torch.Tensor:
     """``F.grouped_mm`` where torch provides it for the device, otherwise the per-group loop it
     stands for (which reads the offsets on the host)."""
-    if _torch_grouped_mm_usable(a):
+    if a.device.type != "cuda":
+        # host tensors (tests, the CPU reference path): torch's CPU grouped_mm rejects some layouts
+        # it could compute; the loop below is as good there
+        if hasattr(F, "grouped_mm"):
+            try:
+                return F.grouped_mm(a, b, offs=offs)
+            except (RuntimeError, NotImplementedError):
+                pass
+    elif _torch_grouped_mm_usable(a):
         return F.grouped_mm(a, b, offs=offs)
     bounds = [0] + offs.tolist()
     if a.dim() == 2 and b.dim() == 3:  # jagged on rows of a

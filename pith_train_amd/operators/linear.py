@@ -18,6 +18,7 @@ from .deepgemm_quantize import (
     fp8cast_blockwise_transpose,
     fp8cast_rowwise_blockwise_transpose,
     fp8cast_rowwise_transpose,
+    transposed_pitch,
 )
 
 # Kept for importers of the reference module (``from ...linear import ARCH_MAJOR``); nothing in
@@ -43,8 +44,15 @@ def _split_k(m: int, n: int, k: int):
     return (splits, split_len) if splits > 1 else (1, k)
 
 
+def _row_pitch(t: torch.Tensor) -> int:
+    """Row pitch in bytes of a 2-D FP8 operand whose rows are contiguous."""
+    assert t.stride(1) == 1 or t.shape[1] <= 1, "FP8 GEMM operands need contiguous rows"
+    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+
+
 def _fp8_gemm_nt(a_fp8, a_scale, b_fp8, b_scale, m: int, n: int, device, dtype) -> torch.Tensor:
-    """out[m, n] = a @ b.T; a: 1x128 scales, b: 128x128 scales."""
+    """out[m, n] = a @ b.T; a: 1x128 scales, b: 128x128 scales.  The operands may be row-padded
+    views (the transposed operands of the quantisers are, for some token counts)."""
     k = a_fp8.shape[1]
     if k % 16:
         # The kernels fetch 16-byte chunks along the reduction dimension.  A ragged length (a
@@ -54,20 +62,24 @@ def _fp8_gemm_nt(a_fp8, a_scale, b_fp8, b_scale, m: int, n: int, device, dtype) 
         a_fp8 = torch.nn.functional.pad(a_fp8.view(torch.uint8), (0, pad)).view(torch.float8_e4m3fn)
         b_fp8 = torch.nn.functional.pad(b_fp8.view(torch.uint8), (0, pad)).view(torch.float8_e4m3fn)
         k += pad
+    lda, ldb = _row_pitch(a_fp8), _row_pitch(b_fp8)
+    if lda % 16 or ldb % 16:
+        a_fp8, b_fp8 = a_fp8.contiguous(), b_fp8.contiguous()
+        lda = ldb = k
     out_dtype = dtype if dtype in (torch.bfloat16, torch.float32) else torch.float32
     out = torch.empty((m, n), device=device, dtype=out_dtype)
     splits, split_len = _split_k(m, n, k)
     if splits > 1:
         partial = torch.empty((splits, m, n), device=device, dtype=torch.float32)
         _lib.call(
-            "pt_gemm_nt_dense_splitk", a_fp8.data_ptr(), a_scale.data_ptr(), b_fp8.data_ptr(), b_scale.data_ptr(),
-            partial.data_ptr(), splits, split_len, m, n, k, _lib.stream_ptr(device),
+            "pt_gemm_nt_dense_splitk_ld", a_fp8.data_ptr(), lda, a_scale.data_ptr(), b_fp8.data_ptr(), ldb,
+            b_scale.data_ptr(), partial.data_ptr(), splits, split_len, m, n, k, _lib.stream_ptr(device),
         )  # fmt: skip
         _lib.call("pt_sum_partials", partial.data_ptr(), splits, m * n, out.data_ptr(), _lib.dtype_code(out_dtype),
                   _lib.stream_ptr(device))  # fmt: skip
         return out if out_dtype == dtype else out.to(dtype)
     _lib.call(
-        "pt_gemm_nt_dense", a_fp8.data_ptr(), a_scale.data_ptr(), b_fp8.data_ptr(),
+        "pt_gemm_nt_dense_ld", a_fp8.data_ptr(), lda, a_scale.data_ptr(), b_fp8.data_ptr(), ldb,
         b_scale.data_ptr(), out.data_ptr(), _lib.dtype_code(out_dtype), m, n, k,
         _lib.stream_ptr(device),
     )  # fmt: skip
@@ -119,7 +131,7 @@ def _define_ops(namespace: str):
         dev = input_2d.device
         return (
             torch.empty((rows, weight.shape[0]), dtype=input_2d.dtype, device=dev),
-            torch.empty((red, rows), dtype=torch.float8_e4m3fn, device=dev),
+            torch.empty_strided((red, rows), (transposed_pitch(rows), 1), dtype=torch.float8_e4m3fn, device=dev),
             torch.empty((-(-red // 128), -(-rows // 128)), dtype=torch.float32, device=dev),
         )
 

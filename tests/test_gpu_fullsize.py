@@ -122,8 +122,9 @@ def test_full_size_dense_weight_gradient_split_over_the_reduction_matches_the_si
         assert _split_k(n_out, n_in, tokens)[0] > 1
         split = _fp8_gemm_nt(gt, gt_s, xt, xt_s, n_out, n_in, "cuda", torch.float32)
         single = torch.empty((n_out, n_in), device="cuda", dtype=torch.float32)
-        _lib.call("pt_gemm_nt_dense", gt.data_ptr(), gt_s.data_ptr(), xt.data_ptr(), xt_s.data_ptr(), single.data_ptr(),
-                  _lib.dtype_code(torch.float32), n_out, n_in, tokens, _lib.stream_ptr("cuda"))
+        assert gt.stride(0) > tokens and xt.stride(0) > tokens, "32768-token transposed operands are row-padded"
+        _lib.call("pt_gemm_nt_dense_ld", gt.data_ptr(), gt.stride(0), gt_s.data_ptr(), xt.data_ptr(), xt.stride(0), xt_s.data_ptr(),
+                  single.data_ptr(), _lib.dtype_code(torch.float32), n_out, n_in, tokens, _lib.stream_ptr("cuda"))
         scale = single.abs().mean().item()
         assert (split - single).abs().max().item() <= 1e-4 * scale * 50, "more than fp32 reordering noise"
         rows = torch.tensor([0, 127, 128, n_out - 1])

@@ -57,6 +57,19 @@ def test_rowwise_colwise(M, N, dtype):
     _eq(got_t[3], ref[3], "ch_scale")
 
 
+def test_transposed_outputs_of_large_token_counts_are_row_padded_views():
+    """The transposed operands of 2048+ tokens (a multiple of 256) come back as views of buffers
+    with one more 128-byte column per row; the padding is never read as data."""
+    D = _ops()
+    x = _mk((4096, 256), 5)
+    _, _, t, _ = D.fp8cast_rowwise_transpose(x.cuda())
+    _, _, bt, _ = D.fp8cast_rowwise_blockwise_transpose(x.cuda())
+    for v in (t, bt):
+        assert v.shape == (256, 4096) and v.stride() == (4096 + 128, 1) and not v.is_contiguous()
+    _, _, t2, _ = D.fp8cast_rowwise_transpose(_mk((300, 256), 6).cuda())
+    assert t2.is_contiguous()
+
+
 def test_rowwise_colwise_all_zero_and_strided():
     D = _ops()
     z = torch.zeros((128, 256), dtype=torch.bfloat16)
@@ -81,7 +94,8 @@ def test_rowwise_kmajor():
         _eq(g, r, w)
 
 
-TRANS = [(128, 128), (128, 256), (256, 256), (64, 256), (7, 300), (1, 128), (256, 7168), (64, 64), (300, 130), (4096, 512)]
+TRANS = [(128, 128), (128, 256), (256, 256), (64, 256), (7, 300), (1, 128), (256, 7168), (64, 64), (300, 130), (4096, 512),
+         (2048, 200), (8192, 384)]  # the last three: token counts whose transposed outputs get a padded row pitch
 
 
 @pytest.mark.parametrize("M,N", TRANS)
