@@ -263,14 +263,15 @@ static int launch_gemm(const GemmArgs& a, hipStream_t stream) {
 
 // PT_GEMM_IMPL overrides the choice of kernel for measurements: "t" = one 128x128 tile per
 // workgroup, "p0" = persistent two-phase kernel, "q0" / "q1" = persistent software-pipelined kernel
-// (8 / 4 waves).  Unset: chosen per call from the shape (below).
-enum { IMPL_UNSET = -3, IMPL_AUTO = -2, IMPL_TILE = -1, IMPL_PIPELINED = 100 };
+// (8 / 4 waves), "r0" = persistent kernel with the row-split loop.  Unset: chosen per call from the shape (below).
+enum { IMPL_UNSET = -3, IMPL_AUTO = -2, IMPL_TILE = -1, IMPL_PIPELINED = 100, IMPL_ROWSPLIT = 200 };
 static int g_impl = IMPL_UNSET;
 static bool parse_impl(const char* e, int& impl) {
   if (!e || !*e || !strcmp(e, "auto")) impl = IMPL_AUTO;
   else if (!strcmp(e, "t")) impl = IMPL_TILE;
   else if (!strcmp(e, "p0")) impl = 0;
   else if (!strcmp(e, "q0") || !strcmp(e, "q1")) impl = IMPL_PIPELINED + (e[1] - '0');
+  else if (!strcmp(e, "r0")) impl = IMPL_ROWSPLIT;
   else return false;
   return true;
 }
@@ -282,20 +283,18 @@ static int gemm_impl() {
   return g_impl;
 }
 
-// The software-pipelined loop overlaps one wave's LDS reads with its own MFMAs but pays a fixed
-// fill/drain of one 128-block per tile, and its tile switch is slower; the two-phase loop is the
-// better one when a tile's reduction is short or the groups are small (few row tiles per group:
-// many half-empty tiles and frequent changes of the b operand).  Crossovers measured on MI355X
-// inside a training step (operands freshly written, i.e. partly cache-resident):
-//   dense      pipelined from K = 512 on (+5 % at 512, +13..20 % from 2048 on)
-//   m-grouped  pipelined for >= 1536 rows per group and K >= 2048 (+3..13 %); below, -1..-9 %
-//   k-grouped  pipelined for >= 6 blocks of 128 rows per group (+0..6 %); at 4.5 blocks, -5..-9 %
-static bool prefer_pipelined(const GemmArgs& g) {
-  switch (g.mode) {
-    case GEMM_DENSE: return g.red >= 512;
-    case GEMM_M_GROUPED: return g.G > 0 && g.red >= 2048 && g.rows_a >= (int64_t)g.G * 1536;
-    default: return g.G > 0 && g.red >= (int64_t)g.G * 128 * 6;
-  }
+// Choice of the persistent kernel, from measurements on MI355X inside a training step (operands
+// freshly written, i.e. partly cache-resident):
+//   m-grouped, k-grouped  the row-split loop: its loads never pause, which matters most where
+//              operands come from HBM (every group has its own b operand), and waves of a half-empty
+//              tile skip their MFMAs.  +1..5 % per layer over the better of the other two.
+//   dense      the software-pipelined loop from K = 512 on (+5 % at 512, +13..20 % from 2048 on
+//              over the two-phase loop, +5..8 % over the row-split loop); below, the two-phase loop,
+//              which has no fill/drain of one 128-block per tile.
+enum { KERNEL_TWO_PHASE, KERNEL_PIPELINED, KERNEL_ROWSPLIT };
+static int preferred_kernel(const GemmArgs& g) {
+  if (g.mode != GEMM_DENSE) return KERNEL_ROWSPLIT;
+  return g.red >= 512 ? KERNEL_PIPELINED : KERNEL_TWO_PHASE;
 }
 
 // The persistent kernels address operands through 32-bit buffer offsets (signed range for the
@@ -320,7 +319,14 @@ static int dispatch_gemm(const GemmArgs& g, hipStream_t stream) {
              "the output (one group's block of it in the k-grouped mode) through 32-bit byte offsets: operands below 2 GiB, "
              "output below 4 GiB");
   if (impl == IMPL_TILE || !fits) return launch_gemm<128, 128, 2, 2>(g, stream);
-  if (impl == IMPL_AUTO) return prefer_pipelined(g) ? launch_gemm_pipelined(g, 0, stream) : launch_gemm_persistent(g, 0, stream);
+  if (impl == IMPL_AUTO) {
+    switch (preferred_kernel(g)) {
+      case KERNEL_ROWSPLIT: return launch_gemm_rowsplit(g, 0, stream);
+      case KERNEL_PIPELINED: return launch_gemm_pipelined(g, 0, stream);
+      default: return launch_gemm_persistent(g, 0, stream);
+    }
+  }
+  if (impl >= IMPL_ROWSPLIT) return launch_gemm_rowsplit(g, impl - IMPL_ROWSPLIT, stream);
   if (impl >= IMPL_PIPELINED) return launch_gemm_pipelined(g, impl - IMPL_PIPELINED, stream);
   return launch_gemm_persistent(g, impl, stream);
 }
@@ -331,7 +337,7 @@ using namespace pt;
 
 extern "C" int pt_gemm_select_kernel(const char* name) {
   int impl;
-  PT_REQUIRE(parse_impl(name, impl), "gemm_select_kernel: unknown kernel '%s' (auto, p0, q0, q1, t)", name);
+  PT_REQUIRE(parse_impl(name, impl), "gemm_select_kernel: unknown kernel '%s' (auto, p0, q0, q1, r0, t)", name);
   g_impl = impl;
   return PT_OK;
 }

@@ -38,5 +38,7 @@ __device__ __forceinline__ int k_group_end(const GemmArgs& p, int g) {
 int launch_gemm_persistent(const GemmArgs& a, int variant, hipStream_t stream);
 // persistent kernel with the software-pipelined main loop (gemm_pipelined.hip)
 int launch_gemm_pipelined(const GemmArgs& a, int variant, hipStream_t stream);
+// persistent kernel whose two steps per 128-block split the tile by rows (gemm_rowsplit.hip)
+int launch_gemm_rowsplit(const GemmArgs& a, int variant, hipStream_t stream);
 
 }  // namespace pt

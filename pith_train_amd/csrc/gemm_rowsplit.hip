@@ -1,0 +1,342 @@
+// Persistent FP8 GEMM for gfx950 whose direct-to-LDS loads are in progress all the time.
+//
+// The loads of a CU move at most ~70 GB/s out of L2: a 64 KiB stage of a 256 x 256 x 128 tile needs
+// about as long to arrive as its MFMAs need to run, so the load path must never idle.  In the
+// two-slot ring of the other persistent kernels a slot can be refilled only after every wave has
+// read all of its fragments, i.e. during one half of the loop body.  Here the two MFMA steps of a
+// 128-block are cut by rows instead of by reduction depth:
+//
+//   step X:  A blocks 0,1 (rows 0-63 of the wave's 128) x B blocks 0,1, both 64-deep halves
+//   step Y:  A blocks 2,3 (rows 64-127)                 x B blocks 0,1, both halves
+//
+// with B block 0 first and B block 1 second inside either step.  A wave then holds, at any time,
+// two A blocks and two B blocks of full depth (96 registers, as before), and the fragments are
+// read in this order: B1 and A2,A3 of block g during X(g); A0,A1 and B0 of block g + 1 during
+// Y(g).  So when X(g) begins, the rows of A0,A1 and B0 of the slot are free (half of it, whole
+// 128-byte lines), and when Y(g) begins the other half is: either step refills the half slot it
+// finds free with the data of block g + 2, 32 KiB per step, requested 1.5 blocks before it is
+// read.  One workgroup barrier per step.
+//
+// Work list, tile table, LDS layout, scale handling and result stores are those of the
+// software-pipelined kernel (gemm_pipelined.hip, gemm_persistent_parts.h).
+#include "gemm_persistent_parts.h"
+#include <type_traits>
+
+namespace pt {
+
+template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC>
+__global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel(GemmArgs p) {
+  constexpr int NW = WGM * WGN;
+  constexpr int WM = BM / WGM, WN = BN / WGN;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  // 128 accumulator values per lane fit next to everything else in the 256 ordinary registers a
+  // wave has at two waves per SIMD; 256 need the accumulation registers.
+  constexpr bool kAccInAgpr = TM * TN * 16 > 128;
+  constexpr int BK = 128;                      // reduction depth of one stage = one scale block = two MFMA steps
+  constexpr int NS = 2;                        // stages in the LDS ring
+  constexpr int STAGE = (BM + BN) * BK;
+  constexpr int SLA = BM / 64, SLB = BN / 64;  // 256 B wave-loads per scale vector
+  static_assert(BM == 256 && BN == 256 && WGM == 2 && WGN == 4, "the row split is written for 8 waves of 128 x 64");
+  constexpr int NP = 5;  // loads a wave issues per step: two 1 KiB loads of a rows, two of b rows, one of scales
+  constexpr int SC_RING = NS;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];  // [NS][STAGE] operand stages | [SC_RING][BM+BN] fp32 scales
+  __shared__ int s_pref[MODE != GEMM_DENSE ? kMaxGroupsGemm + 2 : 2];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+  const uint32_t sc_base = lds_base + NS * STAGE;
+  const float* sc_lds = (const float*)(lds + NS * STAGE);
+
+  // ---- tile list ----
+  int total_tiles;
+  if (MODE == GEMM_M_GROUPED) {
+    scan_group_tiles<BM>(p, s_pref, tid, lane);
+    total_tiles = __builtin_amdgcn_readfirstlane(s_pref[p.G]) * p.tiles_b;
+  } else {
+    total_tiles = (int)p.total_tiles;
+    if (MODE == GEMM_K_GROUPED) scan_group_costs(p, s_pref, tid, lane);
+  }
+  const int xcd = blockIdx.x & 7;
+  // lanes 0 and 1 find the two ends of this XCD's share of the list side by side
+  const int t_step = gridDim.x >> 3;
+  const int t_cut = xcd_first_tile<MODE>(p, s_pref, total_tiles, xcd + (lane & 1), t_step);
+  const int t_end = __builtin_amdgcn_readlane(t_cut, 1);
+  const int t_first = __builtin_amdgcn_readlane(t_cut, 0) + (blockIdx.x >> 3);
+
+  auto decode_any = [&](int t, Tile& T) { decode_tile<MODE, BM, BN>(p, s_pref, t, T); };
+
+  // ---- tile table: the first kTileTable tiles of this workgroup, decoded once by as many lanes
+  // in parallel; the two cursors (loader, MFMAs) then fetch a tile with one LDS read each instead
+  // of redoing the group search and the integer divisions at every tile switch ----
+  constexpr int kTileTable = 48;
+  __shared__ __attribute__((aligned(16))) int s_tiles[kTileTable][8];
+  if (tid < kTileTable) {
+    const int t = t_first + tid * t_step;
+    if (t < t_end) {
+      Tile T;
+      decode_any(t, T);
+      *(int4*)&s_tiles[tid][0] = make_int4(T.a_row0, T.b_row0, T.a_lim, T.b_lim);
+      *(int4*)&s_tiles[tid][4] = make_int4(T.k_begin, T.k_len, T.kb0, T.g);
+    }
+  }
+  __syncthreads();
+  // n = ordinal of the tile in this workgroup's list (t = t_first + n * t_step)
+  auto decode = [&](int n, int t, Tile& T) {
+    if (n < kTileTable) {
+      const int4 a = *(const int4*)&s_tiles[n][0];
+      const int4 b = *(const int4*)&s_tiles[n][4];
+      T.a_row0 = __builtin_amdgcn_readfirstlane(a.x); T.b_row0 = __builtin_amdgcn_readfirstlane(a.y);
+      T.a_lim = __builtin_amdgcn_readfirstlane(a.z); T.b_lim = __builtin_amdgcn_readfirstlane(a.w);
+      T.k_begin = __builtin_amdgcn_readfirstlane(b.x); T.k_len = __builtin_amdgcn_readfirstlane(b.y);
+      T.kb0 = __builtin_amdgcn_readfirstlane(b.z); T.g = __builtin_amdgcn_readfirstlane(b.w);
+    } else {
+      Tile U;
+      decode_any(t, U);
+      T.a_row0 = __builtin_amdgcn_readfirstlane(U.a_row0); T.b_row0 = __builtin_amdgcn_readfirstlane(U.b_row0);
+      T.a_lim = __builtin_amdgcn_readfirstlane(U.a_lim); T.b_lim = __builtin_amdgcn_readfirstlane(U.b_lim);
+      T.k_begin = __builtin_amdgcn_readfirstlane(U.k_begin); T.k_len = __builtin_amdgcn_readfirstlane(U.k_len);
+      T.kb0 = __builtin_amdgcn_readfirstlane(U.kb0); T.g = __builtin_amdgcn_readfirstlane(U.g);
+    }
+  };
+
+  // ---- LDS addressing ----
+  // A stage holds rows of 128 bytes (8 chunks of 16).  Row r keeps logical chunk c at position
+  // c ^ fs(r), fs(r) = (r&7) ^ ((r>>3)&1), which spreads the ds_read_b128 of 8 or 16 consecutive
+  // rows over all banks.  Direct-to-LDS wave-load q covers rows 8q..8q+7 (1 KiB, eight full
+  // 128-byte lines): lane -> row 8q + lane/8, position lane%8, i.e. logical chunk
+  // (lane%8) ^ (lane/8) ^ (q&1).  A wave's loads q = w, w+NW, ... all have the parity of w, so one
+  // per-lane offset serves them all and the rest of the address is uniform (scalar offset).
+  const int chunk = (lane & 7) ^ (lane >> 3) ^ (wave & 1);
+  const uint32_t va = (uint32_t)(lane >> 3) * (uint32_t)p.lda + chunk * 16;
+  const uint32_t vb = (uint32_t)(lane >> 3) * (uint32_t)p.ldb + chunk * 16;
+  const int fs_rd = (lane & 7) ^ ((lane >> 3) & 1);
+  const int roff = (lane & 31) * 128;
+  int coff[2][2];  // [MFMA step][half]: the lane's two chunks of a row for that step
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) coff[ks][h] = roff + (((ks * 4 + (lane >> 5) * 2 + h) ^ fs_rd) << 4);
+
+  const v4i rs_a = make_rsrc(p.a, (uint32_t)p.a_bytes);
+  const v4i rs_sa = make_rsrc(p.sa, (uint32_t)p.sa_bytes);
+
+  // ---- loader: walks (tile, 128-block, half) triples ahead of the MFMAs ----
+  // Half 0 of a block: a rows 128r + 0..63 and b rows 64c + 0..31 (the A0,A1 and B0 fragments of
+  // every wave) plus the block's scales; half 1: the other rows.  Wave-load q covers rows 8q..8q+7.
+  Tile L;
+  int lt = t_first - t_step, l_u = 0, l_nu = 0;  // l_u: next step of the loader's tile, l_nu: its number of steps
+  int l_n = -1, c_n = -1;  // per-cursor ordinal of the current tile in this workgroup's list
+  v4i rs_b = rs_a, rs_sb = rs_sa;
+  uint32_t vs = 0;  // this wave's per-lane scale offset (bytes) at block 0 of the loader's tile
+  bool l_ok = false, l_in = false;
+  int l_half = 0;
+  uint32_t l_sA = 0, l_soA = 0, l_soB = 0, l_sc = 0, l_sa_off = 0, l_sb_off = 0;
+  int l_a_rows = 0;
+  // After the work list is exhausted the pieces still execute (no branches between the MFMAs)
+  // but every lane's offset is out of range, so nothing is fetched; the wave still issues NP
+  // loads per step, which is what the counted waits rely on.
+  int n_steps = 0;  // issue_begin calls so far (real or not): block = n_steps / 2 picks the slot, n_steps % 2 the half
+  auto issue_begin = [&]() {
+    l_ok = false;
+    l_in = false;
+    {
+      const int blk = n_steps >> 1;
+      l_half = n_steps & 1;
+      l_sA = lds_base + (blk % NS) * STAGE;
+      l_sc = sc_base + (blk % NS) * (BM + BN) * 4;
+      ++n_steps;
+    }
+    while (l_u >= l_nu) {
+      lt += t_step;
+      if (lt >= t_end) return;
+      decode(++l_n, lt, L);
+      l_u = 0;
+      l_nu = ((L.k_len + 127) >> 7) * 2;
+      rs_b = make_rsrc(p.b + (MODE == GEMM_M_GROUPED ? (int64_t)L.g * p.b_stride_g : 0), (uint32_t)p.b_bytes);
+      rs_sb = make_rsrc(p.sb + (MODE == GEMM_M_GROUPED ? (int64_t)L.g * p.sb_stride_g : 0), (uint32_t)p.sb_bytes);
+      if (wave < SLA) {
+        const int r = L.a_row0 + 64 * wave + lane;
+        vs = (uint32_t)(((int64_t)(r >> p.sa_shift) * p.sa_rs + (int64_t)L.kb0 * p.sa_ks) * 4);
+      } else {
+        const int r = L.b_row0 + 64 * (wave - SLA) + lane;
+        vs = (uint32_t)(((int64_t)(r >> p.sb_shift) * p.sb_rs + (int64_t)L.kb0 * p.sb_ks) * 4);
+      }
+    }
+    const int l_it = l_u >> 1;
+    const uint32_t koff = (uint32_t)l_it * BK;
+    l_in = (int)(koff + chunk * 16) < L.k_len;  // false only in a ragged last 128-block
+    l_a_rows = L.a_lim - L.a_row0;  // rows past the end of a ragged group are not fetched
+    l_soA = (uint32_t)L.a_row0 * (uint32_t)p.lda + L.k_begin + koff;
+    l_soB = (uint32_t)L.b_row0 * (uint32_t)p.ldb + L.k_begin + koff;
+    l_sa_off = (uint32_t)(l_it * p.sa_ks * 4);
+    l_sb_off = (uint32_t)(l_it * p.sb_ks * 4);
+    l_ok = true;
+    ++l_u;
+  };
+  // Load number k (0 <= k < NP) of the step set up by issue_begin.  The wave-load numbers keep the
+  // parity of the wave (the LDS swizzle of a load depends on it, see above).
+  auto issue_piece = [&](int k) {
+    if (k < 2) {
+      const int q = 16 * k + 8 * l_half + wave;
+      dma16(rs_a, (l_in && 8 * q < l_a_rows) ? va : kOob, l_soA + (uint32_t)(8 * q) * (uint32_t)p.lda, l_sA + q * 1024);
+    } else if (k < 4) {
+      const int q = 8 * (2 * (k - 2) + (wave >> 2)) + 4 * l_half + (wave & 3);
+      dma16(rs_b, l_in ? vb : kOob, l_soB + (uint32_t)(8 * q) * (uint32_t)p.ldb, l_sA + BM * BK + q * 1024);
+    } else {
+      // scales go with the first half of a block; with the second the same instruction is issued
+      // out of range into a sink, so that every step counts the same number of loads
+      const uint32_t sink = sc_base + SC_RING * (BM + BN) * 4;
+      const bool real = l_ok && l_half == 0;
+      if (wave < SLA) dma4(rs_sa, real ? vs : kOob, l_sa_off, real ? l_sc + wave * 256 : sink);
+      else            dma4(rs_sb, real ? vs : kOob, l_sb_off, real ? l_sc + wave * 256 : sink);
+    }
+  };
+  auto issue_step = [&]() {
+    issue_begin();
+#pragma unroll
+    for (int k = 0; k < NP; ++k) issue_piece(k);
+  };
+
+  // one 32-row block of fragments, 64 deep: rows blk_row.. of block `blk` (a: wm0 + 32 i, b: BM + wn0 + 32 j), half ks
+  auto read_frag = [&](int stage, int row0, int ks) -> v8i {
+    const uint8_t* base = lds + (stage % NS) * STAGE + row0 * BK;
+    const uint4 lo = *(const uint4*)(base + coff[ks][0]);
+    const uint4 hi = *(const uint4*)(base + coff[ks][1]);
+    return v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+  };
+  auto a_row = [&](int i) { return wm0 + 32 * i; };
+  auto b_row = [&](int j) { return BM + wn0 + 32 * j; };
+
+#pragma unroll 1
+  for (int s = 0; s < 2 * NS; ++s) issue_step();
+
+  // The E8M0 exponent bytes of a block's scales, packed one byte per 32-row block: the MFMA picks
+  // its byte with the opsel immediates, so a whole block costs two registers.
+  auto read_scales = [&](int stage, int& pa, int& pb) {
+    const float* scA = sc_lds + (stage % NS) * (BM + BN);
+    const float* scB = scA + BM;
+    uint32_t a = 0, b = 0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a |= ((__float_as_uint(scA[wm0 + i * 32 + (lane & 31)]) >> 23) & 0xFFu) << (8 * i);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b |= ((__float_as_uint(scB[wn0 + j * 32 + (lane & 31)]) >> 23) & 0xFFu) << (8 * j);
+    pa = (int)a; pb = (int)b;
+  };
+  // fragments: [block][64-deep half]
+  v8i fa01[2][2], fa23[2][2], fb0[2], fb1[2];
+  int sca = 0, scb = 0, sca_n = 0, scb_n = 0;
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * NP) : "memory");  // the first half of block 0 has landed
+  __syncthreads();
+  read_scales(0, sca, scb);
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    fa01[0][ks] = read_frag(0, a_row(0), ks);
+    fa01[1][ks] = read_frag(0, a_row(1), ks);
+    fb0[ks] = read_frag(0, b_row(0), ks);
+  }
+
+  int gs = 0;  // global 128-block counter: the block the MFMAs consume next
+  Tile C;
+#pragma unroll 1
+  for (int t = t_first; t < t_end; t += t_step) {
+    decode(++c_n, t, C);
+    const int nk = (C.k_len + 127) >> 7;
+    // Waves whose whole row range lies past the end of a ragged group skip the MFMAs, which leaves
+    // the matrix pipe to the other wave of their SIMD, and have nothing to store; they still take
+    // part in the loads, the fragment reads and the barriers.
+    const bool wave_active = C.a_row0 + wm0 < C.a_lim;
+
+    v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+#pragma unroll 1
+    for (int it = 0; it < nk; ++it, ++gs) {
+      // Slot m of a step: MFMA (block row i, block column j, half ks).  The same accumulator comes
+      // back two slots later, not in the next one; B block 1 is first needed in slot 4.
+      //   m:   0        1        2        3        4        5        6        7
+      //   X: (0,0,0)  (1,0,0)  (0,0,1)  (1,0,1)  (0,1,0)  (1,1,0)  (0,1,1)  (1,1,1)
+      //   Y: (2,0,0)  (3,0,0)  (2,0,1)  (3,0,1)  (2,1,0)  (3,1,0)  (2,1,1)  (3,1,1)
+      // ---- step X: this wave's loads of the second half of block gs have landed (only the loads
+      // of the last two steps may be outstanding) and everybody has read the first half ----
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * NP) : "memory");
+      __syncthreads();
+      issue_begin();
+#pragma unroll
+      for (int m = 0; m < 8; ++m) {
+        const int i = m & 1, j = m >> 2, ks = (m >> 1) & 1;
+        if (wave_active) mfma_sel<false>(fa01[i][ks], j ? fb1[ks] : fb0[ks], acc[i][j], i, sca, j, scb);
+#pragma unroll
+        for (int k = m * NP / 8; k < (m + 1) * NP / 8; ++k) issue_piece(k);
+        // fragment reads of this step: B1 first (slots 0, 1), then A2, A3 (slots 2-5)
+        if (m < 2) fb1[m] = read_frag(gs, b_row(1), m);
+        else if (m < 6) fa23[(m - 2) >> 1][(m - 2) & 1] = read_frag(gs, a_row(2 + ((m - 2) >> 1)), (m - 2) & 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // ---- step Y: the first half of block gs + 1 has landed and everybody has read the second
+      // half of block gs ----
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * NP) : "memory");
+      __syncthreads();
+      issue_begin();
+#pragma unroll
+      for (int m = 0; m < 8; ++m) {
+        const int i = m & 1, j = m >> 2, ks = (m >> 1) & 1;
+        if (wave_active) mfma_sel<false>(fa23[i][ks], j ? fb1[ks] : fb0[ks], acc[2 + i][j], 2 + i, sca, j, scb);
+#pragma unroll
+        for (int k = m * NP / 8; k < (m + 1) * NP / 8; ++k) issue_piece(k);
+        // fragment reads for the next block: A0, A1 (slots 0-3), its scales, and B0 once the last
+        // MFMA on the current B0 (slot 3) is two slots behind (slots 5, 6)
+        if (m == 0) read_scales(gs + 1, sca_n, scb_n);
+        if (m < 4) fa01[m >> 1][m & 1] = read_frag(gs + 1, a_row(m >> 1), m & 1);
+        else if (m == 5 || m == 6) fb0[m - 5] = read_frag(gs + 1, b_row(0), m - 5);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      sca = sca_n; scb = scb_n;
+    }
+    // the compiler does not see the MFMAs inside the assembly statements: cover the result latency
+    // of the last one before the epilogue reads the accumulators
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue ----
+    if (!wave_active) continue;
+    if (MODE == GEMM_K_GROUPED && nk == 0 && ACC) continue;
+    store_tile<MODE, TM, TN, ACC, 2>(acc, p, C, wm0, wn0, lane, lds + NS * STAGE + SC_RING * (BM + BN) * 4 + 512 + wave * 2048);
+  }
+  wait_all_vmem();  // nothing may still be writing into this workgroup's LDS when it retires
+}
+
+template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC>
+static int launch_one(GemmArgs a, hipStream_t stream) {
+  // LDS: two operand stages, two stages of scales, a sink line, 2 KiB of result staging per wave
+  constexpr size_t lds = (size_t)2 * (BM + BN) * 128 + 2 * (BM + BN) * 4 + 512 + (size_t)WGM * WGN * 2048;
+  static bool attr_set = false;
+  const int64_t upper = plan_tiles(a, BM, BN);
+  return launch_persistent_grid(fp8_gemm_nt_rowsplit_kernel<MODE, BM, BN, WGM, WGN, ACC>, "fp8_gemm_nt_rowsplit_kernel", a, upper, WGM * WGN * 64, lds, attr_set, stream);
+}
+
+template <int BM, int BN, int WGM, int WGN>
+static int launch_mode(const GemmArgs& a, hipStream_t stream) {
+  switch (a.mode) {
+    case GEMM_DENSE: return launch_one<GEMM_DENSE, BM, BN, WGM, WGN, false>(a, stream);
+    case GEMM_M_GROUPED: return launch_one<GEMM_M_GROUPED, BM, BN, WGM, WGN, false>(a, stream);
+    default:
+      return a.accumulate ? launch_one<GEMM_K_GROUPED, BM, BN, WGM, WGN, true>(a, stream)
+                          : launch_one<GEMM_K_GROUPED, BM, BN, WGM, WGN, false>(a, stream);
+  }
+}
+
+int launch_gemm_rowsplit(const GemmArgs& a, int variant, hipStream_t stream) {
+  PT_REQUIRE(a.mode == GEMM_DENSE || a.G <= kMaxGroupsGemm, "gemm: at most %d groups", kMaxGroupsGemm);
+  switch (variant) {
+    case 0: return launch_mode<256, 256, 2, 4>(a, stream);  // 8 waves, 128 x 64 per wave
+  }
+  PT_REQUIRE(false, "gemm: unknown variant %d", variant);
+}
+
+}  // namespace pt

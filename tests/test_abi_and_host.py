@@ -50,7 +50,7 @@ def test_gemm_kernel_selection_validates_names_without_a_gpu():
     from pith_train_amd import _lib
 
     lib = _lib.load()
-    for name in (b"auto", b"p0", b"q0", b"q1", b"t", None):
+    for name in (b"auto", b"p0", b"q0", b"q1", b"r0", b"t", None):
         assert lib.pt_gemm_select_kernel(name) == 0
     assert lib.pt_gemm_select_kernel(b"fastest") != 0
     assert b"fastest" in lib.pt_last_error()

@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 REL = 1e-2
 
 
-@pytest.fixture(autouse=True, params=["auto", "p0", "q0", "q1", "t"])
+@pytest.fixture(autouse=True, params=["auto", "p0", "q0", "q1", "r0", "t"])
 def gemm_kernel(request):
     """Every test runs once per GEMM kernel of the library (and once with the library's own choice)."""
     from pith_train_amd import _lib
