@@ -29,8 +29,11 @@ HBM_PEAK_GBS = 8000.0
 
 # Average HBM bytes moved by one GEMM launch (fetch + write), from the FETCH_SIZE / WRITE_SIZE
 # counter runs summarised under profiles/ (scaled by the same counters' readings for a plain copy
-# of known size).  None for a workload that has no counter run.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-30b-a3b-moe": 793e6}
+# of known size).  FETCH_SIZE counts what the L2 asks of the fabric, whether the memory-side cache
+# or HBM answers: where successive waves of tiles re-read operand panels that the 4 MiB L2 of an
+# XCD cannot keep (GPT-OSS: 2.5x the algorithmic bytes) most of the excess is served by that cache.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-30b-a3b-moe": 790e6, "dsv2-lite-moe": 488e6, "gpt-oss-20b-moe": 2906e6,
+                                 "qwen3-decoder-linears-32k": 979e6}
 
 WORKLOADS = {
     # name: (kind, hidden, intermediate, experts, top_k, tokens, zipf)
@@ -584,7 +587,7 @@ def main():
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "fp8_gemm_nt_persistent_kernel / fp8_gemm_nt_pipelined_kernel (every GEMM launch of the step: fwd, dgrad, wgrad; the library picks the main loop per shape)",
+            "kernel": "fp8_gemm_nt_rowsplit_kernel (grouped launches) / fp8_gemm_nt_pipelined_kernel (dense launches): every GEMM launch of the step, fwd, dgrad, wgrad; the library picks the main loop per mode and shape",
             "achieved": achieved,
             "peak": FP8_DENSE_PEAK_TFLOPS,
             "unit": "TFLOP/s",
