@@ -258,6 +258,15 @@ def hbm_kernel_report(H, I, E, rows, eidx, top_k=8, kind="fused", extras=None):
                     "GB/s": round(gbs, 0), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 3)})
 
     g = torch.Generator(device="cuda").manual_seed(0)
+    # What this part's memory system gives a kernel that does nothing else: a device-to-device
+    # copy and a fill of 512 MiB (2 x the memory-side cache), by the framework's own kernels.
+    # The fractions of the kernels below are to be read against these, not against 1.0.
+    ref_a = torch.randn((256 << 20,), device="cuda", generator=g).bfloat16()
+    ref_b = torch.empty_like(ref_a)
+    nb = ref_a.numel() * 2
+    rep("reference: device-to-device copy (torch copy_), 512 MiB read + 512 MiB written", timeit(lambda: ref_b.copy_(ref_a)), 2 * nb)
+    rep("reference: fill (torch zero_), 512 MiB written", timeit(lambda: ref_b.zero_()), nb)
+    del ref_a, ref_b
     src = torch.randn((rows, H), device="cuda", generator=g).bfloat16()
     xp, reverse, offs, ks, ks_tensor = TS.scatter_for_grouped_gemm(src, eidx, E)
     Mp = xp.shape[0]
