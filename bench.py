@@ -149,6 +149,7 @@ class GemmTimer:
     """HIP events (on the stream the kernels are launched on) around every GEMM entry point."""
 
     NAMES = ("pt_gemm_m_grouped_nt", "pt_gemm_m_grouped_nt_scatter", "pt_gemm_m_grouped_nt_bias",
+             "pt_gemm_m_grouped_nn", "pt_gemm_m_grouped_nn_scatter",
              "pt_gemm_m_grouped_nt_scatter_bias", "pt_gemm_k_grouped_wgrad",
              "pt_gemm_k_grouped_wgrad_ld",
              "pt_gemm_nt_dense", "pt_gemm_nt_dense_splitk", "pt_gemm_nt_dense_ld", "pt_gemm_nt_dense_splitk_ld")

@@ -131,7 +131,9 @@ int pt_quant_rowwise_blockwise_transpose_ld(const void* x, int dtype, int64_t M,
 /* 128x128 blockwise(x) + blockwise(x^T) for x[G,N,K] (element strides stride_g, stride_row):
  * fp8[G,N,K], scale[G,ceil(N/128),ceil(K/128)], fp8_t[G,K,N], scale_t[G,ceil(K/128),ceil(N/128)].
  * fp8cast_blockwise_transpose (:709-756, G == 1) and fp8cast_blockwise_transpose_batched
- * (:846-899). */
+ * (:846-899).  fp8_t and scale_t may both be NULL: then only fp8 and scale are written (the
+ * transposed twin holds the same bytes and the transposed scale grid, and pt_gemm_m_grouped_nn
+ * reads the forward layout directly). */
 int pt_quant_blockwise_transpose_batched(const void* x, int dtype, int64_t G, int64_t N, int64_t K,
                                          int64_t stride_g, int64_t stride_row, void* fp8,
                                          float* scale, void* fp8_t, float* scale_t,
@@ -193,6 +195,22 @@ int pt_gemm_m_grouped_nt(const void* a_fp8, const float* a_scale, const void* b_
  * token_scatter.py:297-309 (forward) or ScatterForGroupedGemm.backward (:271-284, dgrad) -
  * without the intermediate [M, N] tensor. */
 int pt_gemm_m_grouped_nt_scatter(const void* a_fp8, const float* a_scale, const void* b_fp8,
+                                 const float* b_scale, void* out, int out_dtype,
+                                 const int32_t* offs, int32_t num_groups, int64_t M, int64_t N,
+                                 int64_t K, const int32_t* out_row_index, int64_t out_rows,
+                                 pt_stream_t stream);
+
+/* pt_gemm_m_grouped_nt with the b operand given reduction-major: b[g] is [K, N] (K = the reduction,
+ * row pitch N, N % 16 == 0) with scales [ceil(K/128), ceil(N/128)], i.e. a weight and its
+ * 128 x 128 block scales as the forward pass stores them, read by the input-gradient GEMM
+ * dX = dY W without the transposed FP8 copy of W that the call at grouped_linear.py:192-200 is given
+ * (made by fp8cast_blockwise_transpose_batched, deepgemm_quantize.py:419-456).  Same products, same
+ * order of accumulation, same bits as pt_gemm_m_grouped_nt on the transposed operand.  The _scatter
+ * form stores result row r to out[out_row_index[r], :] like pt_gemm_m_grouped_nt_scatter. */
+int pt_gemm_m_grouped_nn(const void* a_fp8, const float* a_scale, const void* b_fp8,
+                         const float* b_scale, void* out, int out_dtype, const int32_t* offs,
+                         int32_t num_groups, int64_t M, int64_t N, int64_t K, pt_stream_t stream);
+int pt_gemm_m_grouped_nn_scatter(const void* a_fp8, const float* a_scale, const void* b_fp8,
                                  const float* b_scale, void* out, int out_dtype,
                                  const int32_t* offs, int32_t num_groups, int64_t M, int64_t N,
                                  int64_t K, const int32_t* out_row_index, int64_t out_rows,

@@ -45,6 +45,8 @@ SIGNATURES = {
     "pt_gemm_nt_dense_splitk_ld": (c_int, [P, I64, P, P, I64, P, P, I32, I64, I64, I64, I64, P]),
     "pt_sum_partials": (c_int, [P, I32, I64, P, c_int, P]),
     "pt_gemm_m_grouped_nt": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P]),
+    "pt_gemm_m_grouped_nn": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P]),
+    "pt_gemm_m_grouped_nn_scatter": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, I64, P]),
     "pt_gemm_m_grouped_nt_bias": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, P]),
     "pt_gemm_m_grouped_nt_scatter_bias": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, I64, P, P]),
     "pt_gemm_m_grouped_nt_scatter": (c_int, [P, P, P, P, P, c_int, P, I32, I64, I64, I64, P, I64, P]),

@@ -314,6 +314,11 @@ static bool fits_persistent(const GemmArgs& g) {
 static int dispatch_gemm(const GemmArgs& g, hipStream_t stream) {
   const int impl = gemm_impl();
   const bool fits = fits_persistent(g);
+  if (g.b_kmajor) {  // one kernel reads this layout, whatever kernel was selected for the others
+    PT_REQUIRE(fits, "gemm: the reduction-major b operand needs the row-split kernel, which addresses operands below 2 GiB "
+                     "and an output below 4 GiB through 32-bit byte offsets");
+    return launch_gemm_rowsplit(g, 0, stream);
+  }
   PT_REQUIRE((!g.out_row_index && !g.bias) || (impl != IMPL_TILE && fits),
              "gemm: scattered output rows and the fused bias need the persistent kernels, which address every operand and "
              "the output (one group's block of it in the k-grouped mode) through 32-bit byte offsets: operands below 2 GiB, "
@@ -453,7 +458,8 @@ extern "C" int pt_sum_partials(const float* partial, int32_t splits, int64_t n, 
 
 static int gemm_m_grouped_impl(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale, void* out,
                                int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N, int64_t K,
-                               const int32_t* out_row_index, int64_t out_rows, const void* bias, pt_stream_t stream) {
+                               const int32_t* out_row_index, int64_t out_rows, const void* bias, pt_stream_t stream,
+                               bool b_kmajor = false) {
   PT_REQUIRE(M >= 0 && N >= 0 && K >= 0 && G > 0, "gemm_m_grouped_nt: bad sizes");
   if (M == 0 || N == 0) return PT_OK;
   PT_REQUIRE(M % 128 == 0, "gemm_m_grouped_nt: M=%lld must be a multiple of 128", (long long)M);
@@ -472,6 +478,11 @@ static int gemm_m_grouped_impl(const void* a_fp8, const float* a_scale, const vo
   g.a_bytes = M * K; g.b_bytes = N * K; g.sa_bytes = M * KB * 4; g.sb_bytes = NB * KB * 4;
   g.tiles_a = (int)(M / 128); g.tiles_b = (int)NB;
   g.total_tiles = (int64_t)g.tiles_a * g.tiles_b;
+  if (b_kmajor) {
+    // b[g] is [K, N] (row pitch N), its scales [ceil(K/128), ceil(N/128)]: scale(b row n, block kb) = sb[kb * NB + n / 128]
+    PT_REQUIRE(N % 16 == 0, "gemm_m_grouped_nn: N=%lld must be a multiple of 16", (long long)N);
+    g.b_kmajor = 1; g.ldb = N; g.sb_rs = 1; g.sb_ks = NB;
+  }
   if (out_row_index) {
     PT_REQUIRE(out_rows >= 0 && N % 8 == 0 && al16(out) && out_rows * N * 2 < (1ll << 32),
                "gemm_m_grouped_nt_scatter: needs N %% 8 == 0, a 16-byte aligned output smaller than 4 GiB");
@@ -506,6 +517,20 @@ extern "C" int pt_gemm_m_grouped_nt_scatter_bias(const void* a_fp8, const float*
   PT_REQUIRE(out_row_index && bias, "gemm_m_grouped_nt_scatter_bias: null out_row_index or bias");
   return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, out_row_index, out_rows, bias,
                              stream);
+}
+
+extern "C" int pt_gemm_m_grouped_nn(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
+                                    void* out, int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N, int64_t K,
+                                    pt_stream_t stream) {
+  return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, nullptr, 0, nullptr, stream, true);
+}
+
+extern "C" int pt_gemm_m_grouped_nn_scatter(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,
+                                            void* out, int out_dtype, const int32_t* offs, int32_t G, int64_t M, int64_t N,
+                                            int64_t K, const int32_t* out_row_index, int64_t out_rows, pt_stream_t stream) {
+  PT_REQUIRE(out_row_index, "gemm_m_grouped_nn_scatter: null out_row_index");
+  return gemm_m_grouped_impl(a_fp8, a_scale, b_fp8, b_scale, out, out_dtype, offs, G, M, N, K, out_row_index, out_rows, nullptr,
+                             stream, true);
 }
 
 extern "C" int pt_gemm_m_grouped_nt_bias(const void* a_fp8, const float* a_scale, const void* b_fp8, const float* b_scale,

@@ -24,6 +24,7 @@ struct GemmArgs {
   int64_t out_rows;                       // rows of the output when out_row_index is given
   const void* bias;                       // m-grouped only: [G, rows_b] in the output's type, row g added to the rows of group g
   int64_t split_len;                      // k-grouped with offs == null: group g reduces over [g, g + 1) * split_len (split-K)
+  int b_kmajor;                           // m-grouped, row-split kernel: b is [red, rows_b] per group (row pitch ldb) instead of [rows_b, red]
 };
 
 // End of group g's reduction range in the k-grouped mode (its start is the end of group g - 1).

@@ -24,7 +24,9 @@
 
 namespace pt {
 
-template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC>
+// BT: the b operand is given reduction-major, [red][rows_b] with row pitch ldb (the forward layout of
+// a weight, read by its input-gradient GEMM), instead of [rows_b][red].
+template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC, bool BT = false>
 __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel(GemmArgs p) {
   constexpr int NW = WGM * WGN;
   constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -119,6 +121,28 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
 #pragma unroll
     for (int h = 0; h < 2; ++h) coff[ks][h] = roff + (((ks * 4 + (lane >> 5) * 2 + h) ^ fs_rd) << 4);
 
+  // Reduction-major b operand: its part of a stage holds 128 reduction rows of 256 bytes (the
+  // tile's 256 b rows), logical 16-byte chunk c of row k at position c ^ 2 (k & 7): the eight rows
+  // that one transposing read touches put a chunk at eight different positions, and the chunks
+  // c and c + 1 (c even) of the two halves of a 32-row b block never share one, so such a read
+  // spreads over all banks.  A direct-to-LDS
+  // wave-load covers four such rows (lane -> row lane / 16, position lane % 16); a wave's loads are
+  // row quads Q = w, w + 8, ... of a half, so (k & 7) = 4 (w & 1) + lane / 16 for all of them.
+  // Fragments come out of it through the transposing LDS read: in every group of 16 lanes, source
+  // lane s supplies the address of 8 bytes and lane l receives byte (l & 7) of source lanes
+  // (l >> 3), 2 + (l >> 3), ..., 14 + (l >> 3).  With source lane s pointing at reduction row
+  // s / 2 and b rows 8 (s & 1) .. + 7 of the group's 16, lane l gets 8 consecutive reduction
+  // elements of b row l % 16: four such reads are the lane's 32 bytes of an MFMA operand.
+  const int bt_chunk = (lane & 15) ^ (2 * (4 * (wave & 1) + (lane >> 4)));
+  const uint32_t vbt = (uint32_t)(lane >> 4) * (uint32_t)p.ldb + bt_chunk * 16;
+  uint32_t bt_rd[2];  // per b block j: the lane's byte offset inside the b part of a stage, for reduction rows 0-7
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int s16 = lane & 15, g16 = lane >> 4;
+    const int c = (wn0 >> 4) + 2 * j + (g16 & 1);
+    bt_rd[j] = (uint32_t)((32 * (g16 >> 1) + (s16 >> 1)) * 256 + ((c ^ (2 * (s16 >> 1))) << 4) + 8 * (s16 & 1));
+  }
+
   const v4i rs_a = make_rsrc(p.a, (uint32_t)p.a_bytes);
   const v4i rs_sa = make_rsrc(p.sa, (uint32_t)p.sa_bytes);
 
@@ -133,7 +157,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
   bool l_ok = false, l_in = false;
   int l_half = 0;
   uint32_t l_sA = 0, l_soA = 0, l_soB = 0, l_sc = 0, l_sa_off = 0, l_sb_off = 0;
-  int l_a_rows = 0;
+  int l_a_rows = 0, l_koff = 0;
   // After the work list is exhausted the pieces still execute (no branches between the MFMAs)
   // but every lane's offset is out of range, so nothing is fetched; the wave still issues NP
   // loads per step, which is what the counted waits rely on.
@@ -169,7 +193,9 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
     l_in = (int)(koff + chunk * 16) < L.k_len;  // false only in a ragged last 128-block
     l_a_rows = L.a_lim - L.a_row0;  // rows past the end of a ragged group are not fetched
     l_soA = (uint32_t)L.a_row0 * (uint32_t)p.lda + L.k_begin + koff;
-    l_soB = (uint32_t)L.b_row0 * (uint32_t)p.ldb + L.k_begin + koff;
+    l_soB = BT ? (uint32_t)(L.k_begin + koff) * (uint32_t)p.ldb + (uint32_t)L.b_row0
+               : (uint32_t)L.b_row0 * (uint32_t)p.ldb + L.k_begin + koff;
+    l_koff = (int)koff;
     l_sa_off = (uint32_t)(l_it * p.sa_ks * 4);
     l_sb_off = (uint32_t)(l_it * p.sb_ks * 4);
     l_ok = true;
@@ -182,8 +208,16 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
       const int q = 16 * k + 8 * l_half + wave;
       dma16(rs_a, (l_in && 8 * q < l_a_rows) ? va : kOob, l_soA + (uint32_t)(8 * q) * (uint32_t)p.lda, l_sA + q * 1024);
     } else if (k < 4) {
-      const int q = 8 * (2 * (k - 2) + (wave >> 2)) + 4 * l_half + (wave & 3);
-      dma16(rs_b, l_in ? vb : kOob, l_soB + (uint32_t)(8 * q) * (uint32_t)p.ldb, l_sA + BM * BK + q * 1024);
+      if constexpr (BT) {
+        // reduction rows 64 half + 0..63: row quad Q covers rows 4Q..4Q+3; rows past the end of a
+        // ragged reduction are not fetched (they read as zero)
+        const int Q = 16 * l_half + 8 * (k - 2) + wave;
+        const bool in = l_ok && l_koff + 4 * Q + (lane >> 4) < L.k_len;
+        dma16(rs_b, in ? vbt : kOob, l_soB + (uint32_t)(4 * Q) * (uint32_t)p.ldb, l_sA + BM * BK + Q * 1024);
+      } else {
+        const int q = 8 * (2 * (k - 2) + (wave >> 2)) + 4 * l_half + (wave & 3);
+        dma16(rs_b, l_in ? vb : kOob, l_soB + (uint32_t)(8 * q) * (uint32_t)p.ldb, l_sA + BM * BK + q * 1024);
+      }
     } else {
       // scales go with the first half of a block; with the second the same instruction is issued
       // out of range into a sink, so that every step counts the same number of loads
@@ -208,6 +242,26 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
   };
   auto a_row = [&](int i) { return wm0 + 32 * i; };
   auto b_row = [&](int j) { return BM + wn0 + 32 * j; };
+  // The b fragments are kept as fb[late][early]: the half of the b part of a slot that is read
+  // during step X of its block ("late") against the one read ahead during step Y of the block
+  // before.  Row-major b: late = b block j (rows 64c + 32..63), early = 64-deep half.
+  // Reduction-major b: late = the 64-deep half (reduction rows 64..127), early = b block j.
+  auto read_b = [&](int stage, int late, int early) -> v8i {
+    if constexpr (BT) {
+      typedef int v2i_t __attribute__((ext_vector_type(2)));
+      const uint8_t* base = lds + (stage % NS) * STAGE + BM * BK + bt_rd[early] + late * (64 * 256);
+      v8i r;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v2i_t t = __builtin_amdgcn_ds_read_tr8_b64_v2i32((v2i_t __attribute__((address_space(3)))*)(base + q * 8 * 256));
+        r[2 * q] = t[0];
+        r[2 * q + 1] = t[1];
+      }
+      return r;
+    } else {
+      return read_frag(stage, b_row(late), early);
+    }
+  };
 
 #pragma unroll 1
   for (int s = 0; s < 2 * NS; ++s) issue_step();
@@ -225,7 +279,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
     pa = (int)a; pb = (int)b;
   };
   // fragments: [block][64-deep half]
-  v8i fa01[2][2], fa23[2][2], fb0[2], fb1[2];
+  v8i fa01[2][2], fa23[2][2], fb[2][2];
   int sca = 0, scb = 0, sca_n = 0, scb_n = 0;
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * NP) : "memory");  // the first half of block 0 has landed
   __syncthreads();
@@ -234,7 +288,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
   for (int ks = 0; ks < 2; ++ks) {
     fa01[0][ks] = read_frag(0, a_row(0), ks);
     fa01[1][ks] = read_frag(0, a_row(1), ks);
-    fb0[ks] = read_frag(0, b_row(0), ks);
+    fb[0][ks] = read_b(0, 0, ks);
   }
 
   int gs = 0;  // global 128-block counter: the block the MFMAs consume next
@@ -263,6 +317,8 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
       //   m:   0        1        2        3        4        5        6        7
       //   X: (0,0,0)  (1,0,0)  (0,0,1)  (1,0,1)  (0,1,0)  (1,1,0)  (0,1,1)  (1,1,1)
       //   Y: (2,0,0)  (3,0,0)  (2,0,1)  (3,0,1)  (2,1,0)  (3,1,0)  (2,1,1)  (3,1,1)
+      // (with a reduction-major b operand j and ks trade places: both b blocks of the first half,
+      // then both of the second)
       // ---- step X: this wave's loads of the second half of block gs have landed (only the loads
       // of the last two steps may be outstanding) and everybody has read the first half ----
       asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * NP) : "memory");
@@ -270,12 +326,13 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
       issue_begin();
 #pragma unroll
       for (int m = 0; m < 8; ++m) {
-        const int i = m & 1, j = m >> 2, ks = (m >> 1) & 1;
-        if (wave_active) mfma_sel<false>(fa01[i][ks], j ? fb1[ks] : fb0[ks], acc[i][j], i, sca, j, scb);
+        const int i = m & 1, late = m >> 2, early = (m >> 1) & 1;
+        const int j = BT ? early : late, ks = BT ? late : early;
+        if (wave_active) mfma_sel<false>(fa01[i][ks], fb[late][early], acc[i][j], i, sca, j, scb);
 #pragma unroll
         for (int k = m * NP / 8; k < (m + 1) * NP / 8; ++k) issue_piece(k);
         // fragment reads of this step: B1 first (slots 0, 1), then A2, A3 (slots 2-5)
-        if (m < 2) fb1[m] = read_frag(gs, b_row(1), m);
+        if (m < 2) fb[1][m] = read_b(gs, 1, m);
         else if (m < 6) fa23[(m - 2) >> 1][(m - 2) & 1] = read_frag(gs, a_row(2 + ((m - 2) >> 1)), (m - 2) & 1);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -286,15 +343,16 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
       issue_begin();
 #pragma unroll
       for (int m = 0; m < 8; ++m) {
-        const int i = m & 1, j = m >> 2, ks = (m >> 1) & 1;
-        if (wave_active) mfma_sel<false>(fa23[i][ks], j ? fb1[ks] : fb0[ks], acc[2 + i][j], 2 + i, sca, j, scb);
+        const int i = m & 1, late = m >> 2, early = (m >> 1) & 1;
+        const int j = BT ? early : late, ks = BT ? late : early;
+        if (wave_active) mfma_sel<false>(fa23[i][ks], fb[late][early], acc[2 + i][j], 2 + i, sca, j, scb);
 #pragma unroll
         for (int k = m * NP / 8; k < (m + 1) * NP / 8; ++k) issue_piece(k);
         // fragment reads for the next block: A0, A1 (slots 0-3), its scales, and B0 once the last
         // MFMA on the current B0 (slot 3) is two slots behind (slots 5, 6)
         if (m == 0) read_scales(gs + 1, sca_n, scb_n);
         if (m < 4) fa01[m >> 1][m & 1] = read_frag(gs + 1, a_row(m >> 1), m & 1);
-        else if (m == 5 || m == 6) fb0[m - 5] = read_frag(gs + 1, b_row(0), m - 5);
+        else if (m == 5 || m == 6) fb[0][m - 5] = read_b(gs + 1, 0, m - 5);
         __builtin_amdgcn_sched_barrier(0);
       }
       sca = sca_n; scb = scb_n;
@@ -311,20 +369,22 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
   wait_all_vmem();  // nothing may still be writing into this workgroup's LDS when it retires
 }
 
-template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC>
+template <int MODE, int BM, int BN, int WGM, int WGN, bool ACC, bool BT = false>
 static int launch_one(GemmArgs a, hipStream_t stream) {
   // LDS: two operand stages, two stages of scales, a sink line, 2 KiB of result staging per wave
   constexpr size_t lds = (size_t)2 * (BM + BN) * 128 + 2 * (BM + BN) * 4 + 512 + (size_t)WGM * WGN * 2048;
   static bool attr_set = false;
   const int64_t upper = plan_tiles(a, BM, BN);
-  return launch_persistent_grid(fp8_gemm_nt_rowsplit_kernel<MODE, BM, BN, WGM, WGN, ACC>, "fp8_gemm_nt_rowsplit_kernel", a, upper, WGM * WGN * 64, lds, attr_set, stream);
+  return launch_persistent_grid(fp8_gemm_nt_rowsplit_kernel<MODE, BM, BN, WGM, WGN, ACC, BT>, "fp8_gemm_nt_rowsplit_kernel", a, upper, WGM * WGN * 64, lds, attr_set, stream);
 }
 
 template <int BM, int BN, int WGM, int WGN>
 static int launch_mode(const GemmArgs& a, hipStream_t stream) {
   switch (a.mode) {
     case GEMM_DENSE: return launch_one<GEMM_DENSE, BM, BN, WGM, WGN, false>(a, stream);
-    case GEMM_M_GROUPED: return launch_one<GEMM_M_GROUPED, BM, BN, WGM, WGN, false>(a, stream);
+    case GEMM_M_GROUPED:
+      return a.b_kmajor ? launch_one<GEMM_M_GROUPED, BM, BN, WGM, WGN, false, true>(a, stream)
+                        : launch_one<GEMM_M_GROUPED, BM, BN, WGM, WGN, false>(a, stream);
     default:
       return a.accumulate ? launch_one<GEMM_K_GROUPED, BM, BN, WGM, WGN, true>(a, stream)
                           : launch_one<GEMM_K_GROUPED, BM, BN, WGM, WGN, false>(a, stream);
@@ -333,6 +393,7 @@ static int launch_mode(const GemmArgs& a, hipStream_t stream) {
 
 int launch_gemm_rowsplit(const GemmArgs& a, int variant, hipStream_t stream) {
   PT_REQUIRE(a.mode == GEMM_DENSE || a.G <= kMaxGroupsGemm, "gemm: at most %d groups", kMaxGroupsGemm);
+  PT_REQUIRE(!a.b_kmajor || a.mode == GEMM_M_GROUPED, "gemm: a reduction-major b operand is built for the m-grouped mode only");
   switch (variant) {
     case 0: return launch_mode<256, 256, 2, 4>(a, stream);  // 8 waves, 128 x 64 per wave
   }

@@ -15,7 +15,7 @@ namespace pt {
 
 enum { A_ROW = 0, A_BLOCK = 1 };                       // scaling of the same-orientation output
 enum { B_COL = 0, B_BLOCK = 1 };                       // scaling of the twin
-enum { BL_ROWMAJOR = 0, BL_TRANSPOSED = 1, BL_KMAJOR = 2 };  // layout of the twin's bytes
+enum { BL_ROWMAJOR = 0, BL_TRANSPOSED = 1, BL_KMAJOR = 2, BL_NONE = 3 };  // layout of the twin's bytes (BL_NONE: no twin is written)
 enum { BS_MB_N = 0, BS_N_MB = 1 };                     // twin scale layout for B_COL
 
 struct QuantArgs {
@@ -499,6 +499,7 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
 
   // ---- same-orientation output (row-scaled: already written above) ---------------------------
   if (AM != A_ROW) write_same_orientation(blk_scale, blk_rcp);
+  if constexpr (BL == BL_NONE) return;
 
   // ---- twin ---------------------------------------------------------------------------------
   f.fence();
@@ -784,10 +785,10 @@ static int quant_blockwise_transpose_batched_impl(const void* x, int dtype, int6
                                                   pt_stream_t stream) {
   PT_REQUIRE(G >= 0 && N >= 0 && K >= 0 && stride_row >= K, "quant_blockwise_transpose_batched: bad shape");
   if (G == 0 || N == 0 || K == 0) return PT_OK;
-  PT_REQUIRE(x && fp8 && scale && fp8_t && scale_t, "quant_blockwise_transpose_batched: null pointer");
+  PT_REQUIRE(x && fp8 && scale && (fp8_t != nullptr) == (scale_t != nullptr), "quant_blockwise_transpose_batched: null pointer");
   QuantArgs a;
   fill_common(a, x, dtype, N, K, stride_row);
-  PT_REQUIRE(fp8_stride_g >= N * K && t_ld >= N && t_stride_g >= K * t_ld - (t_ld - N) && scale_t_ld >= a.tiles_m,
+  PT_REQUIRE(fp8_stride_g >= N * K && (!fp8_t || (t_ld >= N && t_stride_g >= K * t_ld - (t_ld - N) && scale_t_ld >= a.tiles_m)),
              "quant_blockwise_transpose_batched: output strides smaller than the tensors");
   const int eb = dtype == PT_F32 ? 4 : 2;
   a.vec_in = a.vec_in && ((stride_g * eb) % 16 == 0);
@@ -798,6 +799,7 @@ static int quant_blockwise_transpose_batched_impl(const void* x, int dtype, int6
   // 16-byte transposed stores need every row start aligned: the pitch, the group stride and the base
   a.vec_out_t = a.vec_out_t && (t_ld % 16 == 0) && (t_stride_g % 16 == 0) && (((uintptr_t)fp8_t) % 16 == 0);
   a.vec_out = a.vec_out && (fp8_stride_g % 8 == 0) && (((uintptr_t)fp8) % 8 == 0);
+  if (!fp8_t) return launch_quant<A_BLOCK, B_BLOCK, BL_NONE, BS_MB_N>(a, dtype, G, (hipStream_t)stream);
   return launch_quant<A_BLOCK, B_BLOCK, BL_TRANSPOSED, BS_MB_N>(a, dtype, G, (hipStream_t)stream);
 }
 

@@ -22,7 +22,7 @@ import torch.nn as nn
 from ..dualpipe_utils import FP8WeightCacheControl
 from ..operators import fused_experts
 from ..operators.clamped_swiglu import clamped_swiglu
-from ..operators.deepgemm_quantize import fp8cast_blockwise_transpose_batched, fp8cast_blockwise_transpose_batched_cat
+from ..operators.deepgemm_quantize import fp8cast_grouped_weight, fp8cast_grouped_weight_cat
 from ..operators.grouped_linear import FP8GroupedLinear, FP8GroupedLinearFunc, GroupedLinearFunc
 from ..operators.indexed_bias_add import indexed_bias_add
 from ..operators.silu_mul import silu_mul, silu_mul_halves
@@ -50,10 +50,10 @@ class Qwen3MoeExperts(nn.Module):
         layers' own quantised weights (one quantisation per ``FP8WeightCacheControl`` version)."""
         parts = [self.gate_proj.weight, self.up_proj.weight]
         if torch.compiler.is_compiling():
-            return fp8cast_blockwise_transpose_batched_cat(parts)
+            return fp8cast_grouped_weight_cat(parts)
         ver = FP8WeightCacheControl.version
         if self._gu_cache is None or self._gu_version != ver:
-            self._gu_cache = fp8cast_blockwise_transpose_batched_cat(parts)
+            self._gu_cache = fp8cast_grouped_weight_cat(parts)
             self._gu_version = ver
         return self._gu_cache
 
@@ -156,14 +156,14 @@ class GptOssExperts(nn.Module):
 
     def _quantized_weight(self, name: str, weight: torch.Tensor):
         if torch.compiler.is_compiling():
-            return fp8cast_blockwise_transpose_batched(weight)
+            return fp8cast_grouped_weight(weight)
         ver = FP8WeightCacheControl.version
         cache = self._wq_cache
         if self._wq_version != ver or cache is None:
             cache = self._wq_cache = {}
             self._wq_version = ver
         if name not in cache:
-            cache[name] = fp8cast_blockwise_transpose_batched(weight)
+            cache[name] = fp8cast_grouped_weight(weight)
         return cache[name]
 
     def _group_linear(self, x, weight, name, offs, ks, ks_tensor, group_indices_, in_rows=None, bias=None,

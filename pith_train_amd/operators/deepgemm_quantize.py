@@ -19,6 +19,9 @@ __all__ = [
     "fp8cast_rowwise_blockwise_transpose",
     "fp8cast_blockwise_transpose",
     "fp8cast_blockwise_transpose_batched",
+    "fp8cast_blockwise_batched",
+    "fp8cast_grouped_weight",
+    "fp8cast_grouped_weight_cat",
     "fp8cast_rowwise_colwise_t",
     "fp8cast_rowwise_colwise_t_rows",
 ]
@@ -167,28 +170,28 @@ def fp8cast_rowwise_blockwise_transpose(x: torch.Tensor):
     return out_tok, scale_tok, out_blk_t, scale_blk_t
 
 
-def _blockwise_batched(x3: torch.Tensor):
+def _blockwise_batched(x3: torch.Tensor, twin: bool = True):
     G, N, K = x3.shape
     dev = x3.device
     out = torch.empty((G, N, K), dtype=FP8, device=dev)
     scale = torch.empty((G, _cdiv(N, 128), _cdiv(K, 128)), dtype=torch.float32, device=dev)
-    out_t = torch.empty((G, K, N), dtype=FP8, device=dev)
-    scale_t = torch.empty((G, _cdiv(K, 128), _cdiv(N, 128)), dtype=torch.float32, device=dev)
+    out_t = torch.empty((G, K, N), dtype=FP8, device=dev) if twin else None
+    scale_t = torch.empty((G, _cdiv(K, 128), _cdiv(N, 128)), dtype=torch.float32, device=dev) if twin else None
     if G and N and K:
         _lib.call(
             "pt_quant_blockwise_transpose_batched", x3.data_ptr(), _lib.dtype_code(x3.dtype), G, N, K,
             x3.stride(0) if G > 1 else N * K, x3.stride(1) if N > 1 else K, out.data_ptr(),
-            scale.data_ptr(), out_t.data_ptr(), scale_t.data_ptr(), _lib.stream_ptr(dev),
+            scale.data_ptr(), out_t.data_ptr() if twin else 0, scale_t.data_ptr() if twin else 0, _lib.stream_ptr(dev),
         )  # fmt: skip
     return out, scale, out_t, scale_t
 
 
-def fp8cast_blockwise_transpose_batched_cat(parts):
+def fp8cast_blockwise_transpose_batched_cat(parts, twin: bool = True):
     """:func:`fp8cast_blockwise_transpose_batched` of ``torch.cat(parts, dim=1)`` without the
     concatenation: each ``[G, N_i, K]`` part is quantised straight into its rows of the fused
     outputs (and its columns of the transposed twin).  ``N_i % 128 == 0`` so that the 128x128
     blocks of the fused tensor are blocks of the parts; separate gate and up weights become one
-    fused projection operand this way."""
+    fused projection operand this way.  ``twin=False``: see :func:`fp8cast_blockwise_batched`."""
     G, _, K = parts[0].shape
     dev = parts[0].device
     assert all(p_.ndim == 3 and p_.shape[0] == G and p_.shape[2] == K and p_.shape[1] % 128 == 0 for p_ in parts)
@@ -196,8 +199,8 @@ def fp8cast_blockwise_transpose_batched_cat(parts):
     nb, kb = N // 128, _cdiv(K, 128)
     out = torch.empty((G, N, K), dtype=FP8, device=dev)
     scale = torch.empty((G, nb, kb), dtype=torch.float32, device=dev)
-    out_t = torch.empty((G, K, N), dtype=FP8, device=dev)
-    scale_t = torch.empty((G, kb, nb), dtype=torch.float32, device=dev)
+    out_t = torch.empty((G, K, N), dtype=FP8, device=dev) if twin else None
+    scale_t = torch.empty((G, kb, nb), dtype=torch.float32, device=dev) if twin else None
     row = 0
     for part in parts:
         x3 = _prep2d(part.detach())
@@ -207,7 +210,7 @@ def fp8cast_blockwise_transpose_batched_cat(parts):
                 "pt_quant_blockwise_transpose_batched_into", x3.data_ptr(), _lib.dtype_code(x3.dtype), G, n, K,
                 x3.stride(0) if G > 1 else n * K, x3.stride(1) if n > 1 else K,
                 out.data_ptr() + row * K, N * K, scale.data_ptr() + 4 * (row // 128) * kb, nb * kb,
-                out_t.data_ptr() + row, N, K * N, scale_t.data_ptr() + 4 * (row // 128), nb, kb * nb,
+                out_t.data_ptr() + row if twin else 0, N, K * N, scale_t.data_ptr() + 4 * (row // 128) if twin else 0, nb, kb * nb,
                 _lib.stream_ptr(dev),
             )  # fmt: skip
         row += n
@@ -226,3 +229,33 @@ def fp8cast_blockwise_transpose_batched(x: torch.Tensor):
     """(fp8[G,N,K], scale[G,ceil(N/128),ceil(K/128)], fp8_t[G,K,N], scale_t[G,ceil(K/128),ceil(N/128)])."""
     assert x.ndim == 3, f"Expected 3D tensor, got {x.ndim}D"
     return _blockwise_batched(_prep2d(x.detach()))
+
+
+def fp8cast_blockwise_batched(x: torch.Tensor):
+    """(fp8[G,N,K], scale[G,ceil(N/128),ceil(K/128)], None, None): the first half of
+    :func:`fp8cast_blockwise_transpose_batched`, in the same four-slot tuple.  The transposed twin
+    of a 128x128-blockwise quantisation holds the same bytes and the transposed scale grid; the
+    grouped input-gradient GEMM reads the forward layout directly (``m_grouped_fp8_gemm_nn``), so
+    the grouped-expert weights are quantised without it: a quarter less traffic in this kernel and
+    half the FP8 weight cache."""
+    assert x.ndim == 3, f"Expected 3D tensor, got {x.ndim}D"
+    return _blockwise_batched(_prep2d(x.detach()), twin=False)
+
+
+def weight_twin_enabled() -> bool:
+    """``PITHTRAIN_FP8_WEIGHT_TWIN=1`` keeps the transposed FP8 copy of the grouped-expert weights
+    (the reference's data flow: the input-gradient GEMM then runs in the NT form on it)."""
+    import os
+
+    return os.environ.get("PITHTRAIN_FP8_WEIGHT_TWIN", "0") == "1"
+
+
+def fp8cast_grouped_weight(x: torch.Tensor):
+    """The quantised operand tuple of a grouped-expert weight ``[G, N, K]`` as the grouped linears
+    and fused expert nodes take it: with or without the transposed twin (``weight_twin_enabled``)."""
+    return fp8cast_blockwise_transpose_batched(x) if weight_twin_enabled() else fp8cast_blockwise_batched(x)
+
+
+def fp8cast_grouped_weight_cat(parts):
+    """:func:`fp8cast_grouped_weight` of ``torch.cat(parts, dim=1)`` without the concatenation."""
+    return fp8cast_blockwise_transpose_batched_cat(parts, twin=weight_twin_enabled())

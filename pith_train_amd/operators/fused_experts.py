@@ -15,7 +15,7 @@ import torch
 
 from .. import _lib
 from .deepgemm_quantize import FP8, fp8cast_rowwise_colwise_t, fp8cast_rowwise_colwise_t_rows
-from .grouped_linear import m_grouped_fp8_gemm_nt, schedule_wgrad
+from .grouped_linear import dgrad_operand, m_grouped_fp8_dgrad, m_grouped_fp8_gemm_nt, schedule_wgrad
 from .token_scatter import _GEMM_ALLOC_ALIGNMENT, _PaddedIndexGather
 
 
@@ -153,7 +153,9 @@ def _forward(ctx, x, gate_up_weights, w_down, grouped_mm_offs, q_gate_up, q_down
     h_fp8, h_s, h_ch_t, h_ch_s = silu_mul_quant(gate_up, grouped_mm_offs if row_map is not None else None)
     out = torch.empty((out_m, H), device=x.device, dtype=x.dtype)
     m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, row_map)
-    ctx.save_for_backward(gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, grouped_mm_offs, x_ch_t, x_ch_s,
+    gu_dg, gu_dg_s, ctx.gu_forward_layout = dgrad_operand(q_gate_up)
+    dn_dg, dn_dg_s, ctx.dn_forward_layout = dgrad_operand(q_down)
+    ctx.save_for_backward(gu_dg, gu_dg_s, dn_dg, dn_dg_s, grouped_mm_offs, x_ch_t, x_ch_s,
                           gate_up, h_ch_t, h_ch_s, row_map, expand_idx)
     ctx.gate_up_weights, ctx.w_down = gate_up_weights, w_down
     ctx.rows = (M, out_m, x.shape[0])
@@ -163,23 +165,23 @@ def _forward(ctx, x, gate_up_weights, w_down, grouped_mm_offs, q_gate_up, q_down
 def _backward(ctx, grad_out):
     """Shared backward: returns the gradient of ``x``; the weight gradients go to ``.grad`` (or to
     the ``WeightGradStore`` queue) through :func:`schedule_wgrad`."""
-    (gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, offs, x_ch_t, x_ch_s, gate_up, h_ch_t, h_ch_s,
+    (gu_dg, gu_dg_s, dn_dg, dn_dg_s, offs, x_ch_t, x_ch_s, gate_up, h_ch_t, h_ch_s,
      row_map, expand_idx) = ctx.saved_tensors  # fmt: skip
     M, rows_x, rows_src = ctx.rows
     half = gate_up.shape[1] // 2
-    K = gu_t_fp8.shape[1]
+    K = gu_dg.shape[2] if ctx.gu_forward_layout else gu_dg.shape[1]
     grad_out = grad_out.contiguous()
     if row_map is not None:
         dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t_rows(grad_out, row_map, offs)
     else:
         dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t(grad_out)
     grad_h = torch.empty((M, half), device=grad_out.device, dtype=grad_out.dtype)
-    m_grouped_fp8_gemm_nt((dy_fp8, dy_s), (dn_t_fp8, dn_t_scale), grad_h, offs)
+    m_grouped_fp8_dgrad((dy_fp8, dy_s), dn_dg, dn_dg_s, ctx.dn_forward_layout, grad_h, offs)
     schedule_wgrad(ctx.w_down, (dy_ch_t, dy_ch_s), (h_ch_t, h_ch_s), offs)
     del dy_fp8, dy_s
     dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s = silu_mul_bwd_quant(grad_h, gate_up, offs if row_map is not None else None)
     grad_x = torch.empty((rows_x, K), device=grad_out.device, dtype=grad_out.dtype)
-    m_grouped_fp8_gemm_nt((dgu_fp8, dgu_s), (gu_t_fp8, gu_t_scale), grad_x, offs, row_map)
+    m_grouped_fp8_dgrad((dgu_fp8, dgu_s), gu_dg, gu_dg_s, ctx.gu_forward_layout, grad_x, offs, row_map)
     if expand_idx is not None:
         # one gradient row per routed row so far: rows that expand the same source row are summed
         # (the backward of the expanding gather, token_scatter.py:311-325)
@@ -269,7 +271,9 @@ class FP8ClampedSwiGLUExpertsFunc(torch.autograd.Function):
         out = torch.empty((x.shape[0] if scatter_output else M, H), device=x.device, dtype=x.dtype)
         m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, out_rows,
                               b_down.detach().contiguous())
-        ctx.save_for_backward(gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, grouped_mm_offs, x_ch_t, x_ch_s,
+        gu_dg, gu_dg_s, ctx.gu_forward_layout = dgrad_operand(q_gate_up)
+        dn_dg, dn_dg_s, ctx.dn_forward_layout = dgrad_operand(q_down)
+        ctx.save_for_backward(gu_dg, gu_dg_s, dn_dg, dn_dg_s, grouped_mm_offs, x_ch_t, x_ch_s,
                               gate_up, h_ch_t, h_ch_s, row_map)
         ctx.weights = (w_gate_up, w_down)
         ctx.consts = (float(alpha), float(limit), bool(scatter_output), M, x.shape[0], b_gate_up.dtype, b_down.dtype)
@@ -279,12 +283,12 @@ class FP8ClampedSwiGLUExpertsFunc(torch.autograd.Function):
     def backward(ctx, grad_out):
         from .indexed_bias_add import _segment_sum_along_rows
 
-        (gu_t_fp8, gu_t_scale, dn_t_fp8, dn_t_scale, offs, x_ch_t, x_ch_s, gate_up, h_ch_t, h_ch_s,
+        (gu_dg, gu_dg_s, dn_dg, dn_dg_s, offs, x_ch_t, x_ch_s, gate_up, h_ch_t, h_ch_s,
          row_map) = ctx.saved_tensors  # fmt: skip
         w_gate_up, w_down = ctx.weights
         alpha, limit, scatter_output, M, rows_x, gu_bias_dtype, dn_bias_dtype = ctx.consts
         half = gate_up.shape[1] // 2
-        K = gu_t_fp8.shape[1]
+        K = gu_dg.shape[2] if ctx.gu_forward_layout else gu_dg.shape[1]
         grad_out = grad_out.contiguous()
         out_rows = row_map if scatter_output else None
         if out_rows is not None:
@@ -293,13 +297,13 @@ class FP8ClampedSwiGLUExpertsFunc(torch.autograd.Function):
             dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t(grad_out)
         grad_b_down = _segment_sum_along_rows(grad_out, offs, dn_bias_dtype, out_rows)
         grad_h = torch.empty((M, half), device=grad_out.device, dtype=grad_out.dtype)
-        m_grouped_fp8_gemm_nt((dy_fp8, dy_s), (dn_t_fp8, dn_t_scale), grad_h, offs)
+        m_grouped_fp8_dgrad((dy_fp8, dy_s), dn_dg, dn_dg_s, ctx.dn_forward_layout, grad_h, offs)
         schedule_wgrad(w_down, (dy_ch_t, dy_ch_s), (h_ch_t, h_ch_s), offs)
         del dy_fp8, dy_s
         dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s, col_sum = clamped_swiglu_bwd_quant(grad_h, gate_up, alpha, limit)
         # groups are whole 128-row tiles: their ends in tiles index the per-tile column sums
         grad_b_gate_up = _segment_sum_along_rows(col_sum, offs // 128, gu_bias_dtype)
         grad_x = torch.empty((rows_x if row_map is not None else M, K), device=grad_out.device, dtype=grad_out.dtype)
-        m_grouped_fp8_gemm_nt((dgu_fp8, dgu_s), (gu_t_fp8, gu_t_scale), grad_x, offs, row_map)
+        m_grouped_fp8_dgrad((dgu_fp8, dgu_s), gu_dg, gu_dg_s, ctx.gu_forward_layout, grad_x, offs, row_map)
         schedule_wgrad(w_gate_up, (dgu_ch_t, dgu_ch_s), (x_ch_t, x_ch_s), offs)
         return grad_x, None, grad_b_gate_up, None, grad_b_down, None, None, None, None, None, None, None

@@ -25,7 +25,7 @@ import torch.nn.functional as F
 from .. import _lib
 from ..dualpipe_utils import FP8WeightCacheControl, WeightGradStore
 from .deepgemm_quantize import (
-    fp8cast_blockwise_transpose_batched,
+    fp8cast_grouped_weight,
     fp8cast_rowwise_colwise_t,
     fp8cast_rowwise_colwise_t_rows,
 )
@@ -233,6 +233,48 @@ def schedule_wgrad(weight: torch.Tensor, a_wgrad: tuple, b_wgrad: tuple, offs: t
         grad_weight_fn(a_wgrad, b_wgrad, offs)
 
 
+def m_grouped_fp8_gemm_nn(a, b, out: torch.Tensor, grouped_mm_offs: torch.Tensor,
+                          out_rows: torch.Tensor | None = None) -> torch.Tensor:
+    """out[rows_g] = a[rows_g] @ b[g] with a=(fp8[M,K], scale[M,K/128]) and b=(fp8[G,K,N],
+    scale[G,K/128,N/128]) reduction-major: a weight ``[G, out, in]`` in its forward layout, read by
+    the input-gradient GEMM (K = out features, N = in features).  Same bits as
+    :func:`m_grouped_fp8_gemm_nt` on the transposed operand.  ``out_rows`` as there."""
+    (a_fp8, a_s), (b_fp8, b_s) = a, b
+    M, K = a_fp8.shape
+    G, Kb, N = b_fp8.shape
+    assert Kb == K, (b_fp8.shape, a_fp8.shape)
+    if out_rows is not None:
+        _lib.call(
+            "pt_gemm_m_grouped_nn_scatter", a_fp8.data_ptr(), a_s.data_ptr(), b_fp8.data_ptr(),
+            b_s.data_ptr(), out.data_ptr(), _lib.dtype_code(out.dtype), grouped_mm_offs.data_ptr(), G,
+            M, N, K, out_rows.data_ptr(), out.shape[0], _lib.stream_ptr(out.device),
+        )  # fmt: skip
+        return out
+    _lib.call(
+        "pt_gemm_m_grouped_nn", a_fp8.data_ptr(), a_s.data_ptr(), b_fp8.data_ptr(), b_s.data_ptr(),
+        out.data_ptr(), _lib.dtype_code(out.dtype), grouped_mm_offs.data_ptr(), G, M, N, K,
+        _lib.stream_ptr(out.device),
+    )  # fmt: skip
+    return out
+
+
+def dgrad_operand(quantized_weight: tuple):
+    """(fp8, scale, forward_layout) of the weight operand the input-gradient GEMM reads: the
+    transposed twin when the tuple has one, else the forward-layout tensors themselves."""
+    w_fp8, w_scale, w_t_fp8, w_t_scale = quantized_weight
+    if w_t_fp8 is None:
+        return w_fp8, w_scale, True
+    return w_t_fp8, w_t_scale, False
+
+
+def m_grouped_fp8_dgrad(grad, w_fp8: torch.Tensor, w_scale: torch.Tensor, forward_layout: bool, out: torch.Tensor,
+                        grouped_mm_offs: torch.Tensor, out_rows: torch.Tensor | None = None) -> torch.Tensor:
+    """dX = dY W per group, from whichever weight operand :func:`dgrad_operand` returned."""
+    if forward_layout:
+        return m_grouped_fp8_gemm_nn(grad, (w_fp8, w_scale), out, grouped_mm_offs, out_rows)
+    return m_grouped_fp8_gemm_nt(grad, (w_fp8, w_scale), out, grouped_mm_offs, out_rows)
+
+
 class FP8GroupedLinearFunc(torch.autograd.Function):
     """FP8 grouped linear (grouped_linear.py:104-236): forward and dgrad are m-grouped NT GEMMs on
     1x128-scaled activations against 128x128-scaled weights, wgrad a k-grouped GEMM on the colwise
@@ -280,8 +322,9 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
             bias.detach().contiguous() if bias is not None else None,
         )
         ctx.bias_dtype = bias.dtype if bias is not None else None
+        dg_fp8, dg_scale, ctx.dgrad_forward_layout = dgrad_operand(quantized_weight)
         ctx.save_for_backward(
-            weight_t_fp8, scale_weight_t, grouped_mm_offs, input_ch_t, scale_input_ch, ks_tensor,
+            dg_fp8, dg_scale, grouped_mm_offs, input_ch_t, scale_input_ch, ks_tensor,
             in_rows, out_rows,
         )
         ctx.weight_ref = weight
@@ -292,7 +335,7 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        (weight_t_fp8, scale_weight_t, offs, input_ch_t, scale_input_ch, ks_tensor, in_rows,
+        (dg_fp8, dg_scale, offs, input_ch_t, scale_input_ch, ks_tensor, in_rows,
          out_rows) = ctx.saved_tensors  # fmt: skip
         weight = ctx.weight_ref
         M, K, N, num_groups = ctx.dims
@@ -304,9 +347,7 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
 
         rows_in = ctx.in_m if in_rows is not None else M
         grad_input = torch.empty((rows_in, K), device=grad_output.device, dtype=grad_output.dtype)
-        m_grouped_fp8_gemm_nt(
-            (grad_fp8, scale_grad), (weight_t_fp8, scale_weight_t), grad_input, offs, in_rows
-        )
+        m_grouped_fp8_dgrad((grad_fp8, scale_grad), dg_fp8, dg_scale, ctx.dgrad_forward_layout, grad_input, offs, in_rows)
 
         schedule_wgrad(weight, (grad_ch_t, scale_grad_ch), (input_ch_t, scale_input_ch), offs)
         grad_bias = None
@@ -333,11 +374,11 @@ class FP8GroupedLinear(nn.Module):
 
     def _get_quantized_weight(self):
         if torch.compiler.is_compiling():
-            return fp8cast_blockwise_transpose_batched(self.weight)
+            return fp8cast_grouped_weight(self.weight)
         ver = FP8WeightCacheControl.version
         if self._wq_version == ver and self._wq_cache is not None:
             return self._wq_cache
-        result = fp8cast_blockwise_transpose_batched(self.weight)
+        result = fp8cast_grouped_weight(self.weight)
         self._wq_cache = result
         self._wq_version = ver
         return result

@@ -219,6 +219,42 @@ def test_m_grouped_nt_scattered_rows(sizes, N, K, gemm_kernel):
     assert (out[untouched] == 7.0).all()
 
 
+@pytest.mark.parametrize("sizes,N,K", GROUPED + MANY_GROUPS + [([256], 272, 400), ([600] * 16, 768, 2048)])
+def test_m_grouped_nn_reads_the_forward_layout_weight_with_the_bits_of_nt(sizes, N, K, gemm_kernel):
+    """The input-gradient form: b given reduction-major ([G, K, N], scales [G, K/128, N/128]) is the
+    same product as the NT form on its transpose, accumulated in the same order: equal to the
+    oracle within the GEMM tolerance and to the NT kernel bit for bit, plain and with scattered
+    rows, for ragged N and K too."""
+    from pith_train_amd.operators.grouped_linear import m_grouped_fp8_gemm_nn, m_grouped_fp8_gemm_nt
+
+    ks, offs = _groups(sizes)
+    M, Gn = int(offs[-1]), len(sizes)
+    x = _rand((M, K), M + K + 29)
+    w = _rand((Gn, N, K), N + K + 31, 0.02)
+    a, sa, _, _ = Q.fp8cast_rowwise_colwise(x)
+    b, sb, _, _ = Q.fp8cast_blockwise_transpose_batched(w)
+    ref = G.gemm_m_grouped_nt(a, sa, b, sb, offs, torch.float64)
+    bt, sbt = b.transpose(1, 2).contiguous().cuda(), sb.transpose(1, 2).contiguous().cuda()
+    out_nn = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    out_nt = out_nn.clone()
+    m_grouped_fp8_gemm_nn((a.cuda(), sa.cuda()), (bt, sbt), out_nn, offs.cuda())
+    _check(out_nn, ref, f"m-grouped nn {sizes} N={N} K={K}")
+    if gemm_kernel in ("auto", "r0"):  # the NT launch of the same kernel family
+        m_grouped_fp8_gemm_nt((a.cuda(), sa.cuda()), (b.cuda(), sb.cuda()), out_nt, offs.cuda())
+        assert torch.equal(out_nn[: int(offs[-1])], out_nt[: int(offs[-1])])
+    if N % 8 == 0:
+        g = torch.Generator().manual_seed(M + 1)
+        dst = torch.randperm(M + 5, generator=g)[:M].to(torch.int32)
+        dst[::7] = -1  # dropped rows
+        out_s = torch.full((M + 5, N), 7.0, dtype=torch.bfloat16, device="cuda")
+        m_grouped_fp8_gemm_nn((a.cuda(), sa.cuda()), (bt, sbt), out_s, offs.cuda(), dst.cuda())
+        keep = (dst >= 0).nonzero().flatten()
+        assert torch.equal(out_s[dst[keep].long().cuda()], out_nn[keep.cuda()])
+        untouched = torch.ones(M + 5, dtype=torch.bool)
+        untouched[dst[keep].long()] = False
+        assert (out_s.cpu()[untouched] == 7.0).all()
+
+
 def test_m_grouped_nt_with_more_tiles_per_workgroup_than_the_tile_table_holds(gemm_kernel):
     """Four groups of 25600 rows x 8192 columns: 12800 tiles, 50 per workgroup, so the grouped
     tile decode (group search, row tile inside the group) also runs on the fly for the last tiles.

@@ -444,3 +444,32 @@ def test_moe_combine_without_a_residual_is_the_rounded_weighted_sum():
     got = moe_combine(moe.cuda(), wgt.cuda())
     want = OC.combine_fwd(moe, wgt, torch.zeros((T, H), dtype=torch.bfloat16))
     assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("fuse_permute", [True, False])
+@pytest.mark.parametrize("kind", ["fused", "split", "gpt_oss"])
+def test_stage3_with_and_without_the_transposed_weight_twin_agree_bit_for_bit(kind, fuse_permute, monkeypatch):
+    """PITHTRAIN_FP8_WEIGHT_TWIN=1 keeps the reference's data flow (transposed FP8 weights, NT
+    input-gradient GEMM); the default reads the forward-layout weights in the NN form.  Outputs and
+    all gradients are the same bits."""
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules.experts import forward_stage3
+
+    E, H, I, T, k = 8, 256, 384, 900, 2
+    ids = OM.make_routing(T, E, k, seed=2).reshape(-1).cuda()
+    w = _weights(kind, E, H, I, 3)
+    g = torch.Generator().manual_seed(4)
+    x0 = torch.randn((T * k, H), generator=g).bfloat16().cuda()
+    dy = torch.randn((T * k, H), generator=g).bfloat16().cuda()
+
+    def run(twin):
+        monkeypatch.setenv("PITHTRAIN_FP8_WEIGHT_TWIN", "1" if twin else "0")
+        mod, params = _build(kind, E, H, I, w)
+        FP8WeightCacheControl.step()
+        x = x0.clone().requires_grad_(True)
+        out = forward_stage3(mod, x, ids, E, fuse_permute=fuse_permute)
+        out.backward(dy)
+        return [out.detach(), x.grad] + [p.grad for p in params.values()]
+
+    a, b = run(True), run(False)
+    assert len(a) == len(b) and all(torch.equal(u, v) for u, v in zip(a, b))

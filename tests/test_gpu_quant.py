@@ -263,3 +263,24 @@ def test_clamped_swiglu_fused_into_the_quantisation_has_the_bits_of_the_two_step
     assert col_sum.shape == want.shape
     assert ((col_sum.double() - want).abs() <= 1e-6 * mag + 1e-30).all()
     assert (gate_up.grad == 0).any() and (gate_up.grad != 0).any()  # both sides of the clamps occur
+
+
+@pytest.mark.parametrize("G,N,K", [(3, 256, 384), (2, 200, 300), (1, 128, 128), (4, 1536, 2048)])
+def test_blockwise_batched_without_the_twin_is_the_first_half_of_the_transposing_quantiser(G, N, K):
+    """The grouped-expert weights are quantised without the transposed twin (the input-gradient
+    GEMM reads the forward layout): bytes and scales equal those of the quantiser that writes
+    both, and the fused gate/up form agrees with the concatenation."""
+    from pith_train_amd.operators import deepgemm_quantize as D
+
+    w = (torch.randn((G, N, K), generator=torch.Generator().manual_seed(G + N + K)) * 0.02).bfloat16().cuda()
+    full = D.fp8cast_blockwise_transpose_batched(w)
+    half = D.fp8cast_blockwise_batched(w)
+    assert half[2] is None and half[3] is None
+    assert torch.equal(half[0].view(torch.uint8), full[0].view(torch.uint8)) and torch.equal(half[1], full[1])
+    # the twin of a 128x128-blockwise quantisation is the byte transpose with the transposed scale grid
+    assert torch.equal(full[2].view(torch.uint8), full[0].view(torch.uint8).transpose(1, 2))
+    assert torch.equal(full[3], full[1].transpose(1, 2))
+    if N % 256 == 0:
+        parts = (w[:, : N // 2].contiguous(), w[:, N // 2 :].contiguous())
+        cat = D.fp8cast_blockwise_transpose_batched_cat(parts, twin=False)
+        assert cat[2] is None and torch.equal(cat[0].view(torch.uint8), full[0].view(torch.uint8)) and torch.equal(cat[1], full[1])
