@@ -316,7 +316,8 @@ static int dispatch_gemm(const GemmArgs& g, hipStream_t stream) {
   const bool fits = fits_persistent(g);
   if (g.b_kmajor) {  // one kernel reads this layout, whatever kernel was selected for the others
     PT_REQUIRE(fits, "gemm: the reduction-major b operand needs the row-split kernel, which addresses operands below 2 GiB "
-                     "and an output below 4 GiB through 32-bit byte offsets");
+                     "and an output below 4 GiB through 32-bit byte offsets; larger problems take the NT entry point on the "
+                     "transposed operand");
     return launch_gemm_rowsplit(g, 0, stream);
   }
   PT_REQUIRE((!g.out_row_index && !g.bias) || (impl != IMPL_TILE && fits),

@@ -271,6 +271,8 @@ def m_grouped_fp8_dgrad(grad, w_fp8: torch.Tensor, w_scale: torch.Tensor, forwar
                         grouped_mm_offs: torch.Tensor, out_rows: torch.Tensor | None = None) -> torch.Tensor:
     """dX = dY W per group, from whichever weight operand :func:`dgrad_operand` returned."""
     if forward_layout:
+        # (the NN form exists in the kernel with 32-bit offsets only: a gradient of 2 GiB or an
+        # output of 4 GiB and more needs PITHTRAIN_FP8_WEIGHT_TWIN=1, and the library says so)
         return m_grouped_fp8_gemm_nn(grad, (w_fp8, w_scale), out, grouped_mm_offs, out_rows)
     return m_grouped_fp8_gemm_nt(grad, (w_fp8, w_scale), out, grouped_mm_offs, out_rows)
 
