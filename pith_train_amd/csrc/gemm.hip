@@ -482,6 +482,8 @@ static int gemm_m_grouped_impl(const void* a_fp8, const float* a_scale, const vo
   if (b_kmajor) {
     // b[g] is [K, N] (row pitch N), its scales [ceil(K/128), ceil(N/128)]: scale(b row n, block kb) = sb[kb * NB + n / 128]
     PT_REQUIRE(N % 16 == 0, "gemm_m_grouped_nn: N=%lld must be a multiple of 16", (long long)N);
+    // (b_bytes = K * N is the exact extent of one group's matrix: the kernel leaves the rows past
+    // the end of a ragged reduction to the buffer descriptor's range check)
     g.b_kmajor = 1; g.ldb = N; g.sb_rs = 1; g.sb_ks = NB;
   }
   if (out_row_index) {

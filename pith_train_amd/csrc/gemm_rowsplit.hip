@@ -157,7 +157,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
   bool l_ok = false, l_in = false;
   int l_half = 0;
   uint32_t l_sA = 0, l_soA = 0, l_soB = 0, l_sc = 0, l_sa_off = 0, l_sb_off = 0;
-  int l_a_rows = 0, l_koff = 0;
+  int l_a_rows = 0;
   // After the work list is exhausted the pieces still execute (no branches between the MFMAs)
   // but every lane's offset is out of range, so nothing is fetched; the wave still issues NP
   // loads per step, which is what the counted waits rely on.
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
     l_soA = (uint32_t)L.a_row0 * (uint32_t)p.lda + L.k_begin + koff;
     l_soB = BT ? (uint32_t)(L.k_begin + koff) * (uint32_t)p.ldb + (uint32_t)L.b_row0
                : (uint32_t)L.b_row0 * (uint32_t)p.ldb + L.k_begin + koff;
-    l_koff = (int)koff;
+
     l_sa_off = (uint32_t)(l_it * p.sa_ks * 4);
     l_sb_off = (uint32_t)(l_it * p.sb_ks * 4);
     l_ok = true;
@@ -209,11 +209,12 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
       dma16(rs_a, (l_in && 8 * q < l_a_rows) ? va : kOob, l_soA + (uint32_t)(8 * q) * (uint32_t)p.lda, l_sA + q * 1024);
     } else if (k < 4) {
       if constexpr (BT) {
-        // reduction rows 64 half + 0..63: row quad Q covers rows 4Q..4Q+3; rows past the end of a
-        // ragged reduction are not fetched (they read as zero)
+        // reduction rows 64 half + 0..63: row quad Q covers rows 4Q..4Q+3.  Rows past the end of a
+        // ragged reduction lie past the end of the group's b matrix, whose extent is the
+        // descriptor's: the hardware returns zeros for them (its range check includes the scalar
+        // offset), so no lane needs a check of its own.
         const int Q = 16 * l_half + 8 * (k - 2) + wave;
-        const bool in = l_ok && l_koff + 4 * Q + (lane >> 4) < L.k_len;
-        dma16(rs_b, in ? vbt : kOob, l_soB + (uint32_t)(4 * Q) * (uint32_t)p.ldb, l_sA + BM * BK + Q * 1024);
+        dma16(rs_b, l_ok ? vbt : kOob, l_soB + (uint32_t)(4 * Q) * (uint32_t)p.ldb, l_sA + BM * BK + Q * 1024);
       } else {
         const int q = 8 * (2 * (k - 2) + (wave >> 2)) + 4 * l_half + (wave & 3);
         dma16(rs_b, l_in ? vb : kOob, l_soB + (uint32_t)(8 * q) * (uint32_t)p.ldb, l_sA + BM * BK + q * 1024);
