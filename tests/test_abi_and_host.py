@@ -78,6 +78,24 @@ def test_fused_gemm_stores_refuse_outputs_beyond_the_32_bit_store_offsets():
     assert rc != 0 and b"4 GiB" in lib.pt_last_error()
 
 
+def test_reduction_major_gemm_validates_its_operand_on_the_host():
+    """pt_gemm_m_grouped_nn reads b[g] as [K, N] through 16-byte chunks of its rows and exists only
+    in the kernel with 32-bit offsets: a row length that is not a multiple of 16 and an output of
+    4 GiB or more are refused before any launch (the pointers below are never dereferenced)."""
+    from pith_train_amd import _lib
+
+    lib = _lib.load()
+    p = ctypes.c_void_p(0x10000)
+    I64, I32 = ctypes.c_int64, ctypes.c_int32
+    lib.pt_gemm_m_grouped_nn.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int, ctypes.c_void_p, I32, I64, I64, I64, ctypes.c_void_p]
+    assert lib.pt_gemm_m_grouped_nn(p, p, p, p, p, 0, p, 2, 256, 24, 128, None) != 0
+    assert b"multiple of 16" in lib.pt_last_error()
+    M, N, K = 128 * 20000, 1024, 128  # bf16 output 5.2 GB
+    assert lib.pt_gemm_m_grouped_nn(p, p, p, p, p, 0, p, 4, M, N, K, None) != 0
+    assert b"row-split kernel" in lib.pt_last_error() and b"NT entry point" in lib.pt_last_error()
+    assert lib.pt_gemm_m_grouped_nn(p, p, p, p, p, 0, p, 4, 0, N, K, None) == 0  # nothing to do
+
+
 def test_operators_refuse_cpu_tensors_loudly():
     from pith_train_amd import _lib
     from pith_train_amd.operators.deepgemm_quantize import fp8cast_rowwise_colwise
