@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0
 # or HBM answers: where successive waves of tiles re-read operand panels that the 4 MiB L2 of an
 # XCD cannot keep (GPT-OSS: 2.5x the algorithmic bytes) most of the excess is served by that cache.
 GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-30b-a3b-moe": 792e6, "dsv2-lite-moe": 489e6, "gpt-oss-20b-moe": 2907e6,
-                                 "qwen3-decoder-linears-32k": 971e6}
+                                 "qwen3-decoder-linears-32k": 974e6}
 
 WORKLOADS = {
     # name: (kind, hidden, intermediate, experts, top_k, tokens, zipf)
