@@ -9,13 +9,17 @@
 //   step X:  A blocks 0,1 (rows 0-63 of the wave's 128) x B blocks 0,1, both 64-deep halves
 //   step Y:  A blocks 2,3 (rows 64-127)                 x B blocks 0,1, both halves
 //
-// with B block 0 first and B block 1 second inside either step.  A wave then holds, at any time,
-// two A blocks and two B blocks of full depth (96 registers, as before), and the fragments are
-// read in this order: B1 and A2,A3 of block g during X(g); A0,A1 and B0 of block g + 1 during
-// Y(g).  So when X(g) begins, the rows of A0,A1 and B0 of the slot are free (half of it, whole
-// 128-byte lines), and when Y(g) begins the other half is: either step refills the half slot it
-// finds free with the data of block g + 2, 32 KiB per step, requested 1.5 blocks before it is
-// read.  One workgroup barrier per step.
+// and a ring slot is cut the same way: its half E holds the a rows of block rows 0,1 and one half
+// of the b part (plus the block's scales), its half O the a rows of block rows 2,3 and the other
+// half of the b part.  Inside a step the first 64-deep half comes before the second, which makes
+// the a fragments short-lived: four 8-register buffers hold the step's two block rows x two
+// halves, and each buffer takes a fragment of the next step as soon as the last MFMA on its old
+// content has issued.  With the four b fragments of the block that is 64 fragment registers (the
+// first version of this loop held every fragment of a step before the step began, 96 registers,
+// and spilled), which leaves the compiler a few registers in hand in all variants.  E of block g
+// has been read completely when X(g) ends, O(g) when Y(g) ends; either step refills the half it
+// finds free with block g + 2's data, 32 KiB per step, requested two steps before the barrier
+// behind which it is first read.  One workgroup barrier per step.
 //
 // Work list, tile table, LDS layout, scale handling and result stores are those of the
 // software-pipelined kernel (gemm_pipelined.hip, gemm_persistent_parts.h).
@@ -265,7 +269,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
   };
 
 #pragma unroll 1
-  for (int s = 0; s < 2 * NS; ++s) issue_step();
+  for (int s = 0; s < 2 * NS - 1; ++s) issue_step();
 
   // The E8M0 exponent bytes of a block's scales, packed one byte per 32-row block: the MFMA picks
   // its byte with the opsel immediates, so a whole block costs two registers.
@@ -279,18 +283,18 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
     for (int j = 0; j < TN; ++j) b |= ((__float_as_uint(scB[wn0 + j * 32 + (lane & 31)]) >> 23) & 0xFFu) << (8 * j);
     pa = (int)a; pb = (int)b;
   };
-  // fragments: [block][64-deep half]
-  v8i fa01[2][2], fa23[2][2], fb[2][2];
+  // Fragments.  A: four buffers; the step in progress owns all four (two block rows x two 64-deep
+  // halves) and hands each to the next step's fragment as soon as its last MFMA has issued.  B:
+  // fb[late][early], both block columns and both halves of the current 128-block.
+  v8i fa[4], fb[2][2];
   int sca = 0, scb = 0, sca_n = 0, scb_n = 0;
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * NP) : "memory");  // the first half of block 0 has landed
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NP) : "memory");  // both halves of block 0 have landed
   __syncthreads();
   read_scales(0, sca, scb);
-#pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {
-    fa01[0][ks] = read_frag(0, a_row(0), ks);
-    fa01[1][ks] = read_frag(0, a_row(1), ks);
-    fb[0][ks] = read_b(0, 0, ks);
-  }
+  fa[0] = read_frag(0, a_row(0), 0);
+  fa[1] = read_frag(0, a_row(1), 0);
+  fb[0][0] = read_b(0, 0, 0);
+  fb[0][1] = read_b(0, 0, 1);
 
   int gs = 0;  // global 128-block counter: the block the MFMAs consume next
   Tile C;
@@ -313,47 +317,60 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
 
 #pragma unroll 1
     for (int it = 0; it < nk; ++it, ++gs) {
-      // Slot m of a step: MFMA (block row i, block column j, half ks).  The same accumulator comes
-      // back two slots later, not in the next one; B block 1 is first needed in slot 4.
+      // Slot m of a step: MFMA (block row i, block column j, half ks), the first 64-deep half
+      // before the second:
       //   m:   0        1        2        3        4        5        6        7
-      //   X: (0,0,0)  (1,0,0)  (0,0,1)  (1,0,1)  (0,1,0)  (1,1,0)  (0,1,1)  (1,1,1)
-      //   Y: (2,0,0)  (3,0,0)  (2,0,1)  (3,0,1)  (2,1,0)  (3,1,0)  (2,1,1)  (3,1,1)
-      // (with a reduction-major b operand j and ks trade places: both b blocks of the first half,
-      // then both of the second)
-      // ---- step X: this wave's loads of the second half of block gs have landed (only the loads
-      // of the last two steps may be outstanding) and everybody has read the first half ----
-      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * NP) : "memory");
+      //   X: (0,0,0)  (1,0,0)  (0,1,0)  (1,1,0)  (0,0,1)  (1,0,1)  (0,1,1)  (1,1,1)
+      //   Y: (2,0,0)  (3,0,0)  (2,1,0)  (3,1,0)  (2,0,1)  (3,0,1)  (2,1,1)  (3,1,1)
+      // The same accumulator comes back four slots later.  A fragment (i, ks) of the step lives in
+      // fa[2 ks + (i & 1)] and is used in slots 4 ks + (i & 1) and 4 ks + 2 + (i & 1): the first
+      // half's buffers are free from slot 4 on and take the next step's first-half fragments
+      // (slots 5, 6); the second half's are free when the step ends and take the next step's
+      // second-half fragments in its slots 1, 2.  B fragments fb[late][early] (row-major b: late =
+      // block column, early = half; reduction-major b: the other way round): the "early" part of a
+      // block's slot is read during step Y of the block before (fb[0][.], each after its last MFMA),
+      // the "late" part in slots 0, 1 of step X (fb[1][.]).
+      // The two halves of a ring slot: E = a rows of block rows 0,1 + the early b part (+ scales),
+      // O = a rows of block rows 2,3 + the late b part.  E of block g has been read when X(g) ends
+      // and is refilled during Y(g) with block g + 2; O(g) has been read when Y(g) ends and is
+      // refilled during X(g + 1).  Every refill is requested two steps before the barrier behind
+      // which it is first read, so a step waits until only the previous step's loads are outstanding.
+      // ---- step X ----
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(NP) : "memory");
       __syncthreads();
       issue_begin();
 #pragma unroll
       for (int m = 0; m < 8; ++m) {
-        const int i = m & 1, late = m >> 2, early = (m >> 1) & 1;
-        const int j = BT ? early : late, ks = BT ? late : early;
-        if (wave_active) mfma_sel<false>(fa01[i][ks], fb[late][early], acc[i][j], i, sca, j, scb);
+        const int i = m & 1, j = (m >> 1) & 1, ks = m >> 2;
+        const int late = BT ? ks : j, early = BT ? j : ks;
+        if (wave_active) mfma_sel<false>(fa[2 * ks + i], fb[late][early], acc[i][j], i, sca, j, scb);
 #pragma unroll
         for (int k = m * NP / 8; k < (m + 1) * NP / 8; ++k) issue_piece(k);
-        // fragment reads of this step: B1 first (slots 0, 1), then A2, A3 (slots 2-5)
-        if (m < 2) fb[1][m] = read_b(gs, 1, m);
-        else if (m < 6) fa23[(m - 2) >> 1][(m - 2) & 1] = read_frag(gs, a_row(2 + ((m - 2) >> 1)), (m - 2) & 1);
+        if (m == 0) fb[1][0] = read_b(gs, 1, 0);
+        if (m == 1) { fb[1][1] = read_b(gs, 1, 1); fa[2] = read_frag(gs, a_row(0), 1); }
+        if (m == 2) fa[3] = read_frag(gs, a_row(1), 1);
+        if (m == 5) fa[0] = read_frag(gs, a_row(2), 0);
+        if (m == 6) fa[1] = read_frag(gs, a_row(3), 0);
         __builtin_amdgcn_sched_barrier(0);
       }
-      // ---- step Y: the first half of block gs + 1 has landed and everybody has read the second
-      // half of block gs ----
-      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * NP) : "memory");
+      // ---- step Y ----
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(NP) : "memory");
       __syncthreads();
       issue_begin();
 #pragma unroll
       for (int m = 0; m < 8; ++m) {
-        const int i = m & 1, late = m >> 2, early = (m >> 1) & 1;
-        const int j = BT ? early : late, ks = BT ? late : early;
-        if (wave_active) mfma_sel<false>(fa23[i][ks], fb[late][early], acc[2 + i][j], 2 + i, sca, j, scb);
+        const int i = m & 1, j = (m >> 1) & 1, ks = m >> 2;
+        const int late = BT ? ks : j, early = BT ? j : ks;
+        if (wave_active) mfma_sel<false>(fa[2 * ks + i], fb[late][early], acc[2 + i][j], 2 + i, sca, j, scb);
 #pragma unroll
         for (int k = m * NP / 8; k < (m + 1) * NP / 8; ++k) issue_piece(k);
-        // fragment reads for the next block: A0, A1 (slots 0-3), its scales, and B0 once the last
-        // MFMA on the current B0 (slot 3) is two slots behind (slots 5, 6)
         if (m == 0) read_scales(gs + 1, sca_n, scb_n);
-        if (m < 4) fa01[m >> 1][m & 1] = read_frag(gs + 1, a_row(m >> 1), m & 1);
-        else if (m == 5 || m == 6) fb[0][m - 5] = read_b(gs + 1, 0, m - 5);
+        if (m == 1) fa[2] = read_frag(gs, a_row(2), 1);
+        if (m == 2) fa[3] = read_frag(gs, a_row(3), 1);
+        if (m == 3) fb[0][0] = read_b(gs + 1, 0, 0);
+        if (m == (BT ? 5 : 6)) fb[0][1] = read_b(gs + 1, 0, 1);
+        if (m == 5) fa[0] = read_frag(gs + 1, a_row(0), 0);
+        if (m == 6) fa[1] = read_frag(gs + 1, a_row(1), 0);
         __builtin_amdgcn_sched_barrier(0);
       }
       sca = sca_n; scb = scb_n;

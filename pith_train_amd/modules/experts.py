@@ -184,6 +184,12 @@ class GptOssExperts(nn.Module):
                 and self.gate_up_proj_bias.dtype == x.dtype and self.down_proj_bias.dtype == x.dtype
                 and self.gate_up_proj.shape[1] % 8 == 0 and self.down_proj.shape[1] % 8 == 0)
 
+    def one_node(self, x) -> bool:
+        """Whether the block runs as one autograd node (fused biases and activation).  That node
+        takes every row count from ``grouped_mm_offs`` on the device, so its ``row_map`` may be
+        sized for more rows than the routing produced."""
+        return self.bias_fusable(x) and self.fuse_activation and self.down_proj.shape[2] % 8 == 0
+
     def forward(self, x, grouped_mm_offs, ks=None, ks_tensor=None, row_map=None, scatter_output: bool = False):
         """``row_map`` (extension, FP8 only): the scatter's int32 source-row map; ``x`` is then the
         un-permuted token tensor and the first quantisation gathers its rows.  The result stays
@@ -195,7 +201,7 @@ class GptOssExperts(nn.Module):
         M = x.shape[0] if row_map is None else row_map.shape[0]
         fused = self.bias_fusable(x)
         assert not scatter_output or (fused and row_map is not None), "scatter_output needs row_map and the fused biases"
-        if fused and self.fuse_activation and M % 128 == 0 and self.down_proj.shape[2] % 8 == 0:
+        if M % 128 == 0 and self.one_node(x):
             return fused_experts.FP8ClampedSwiGLUExpertsFunc.apply(
                 x, self.gate_up_proj, self.gate_up_proj_bias, self.down_proj, self.down_proj_bias, grouped_mm_offs,
                 self._quantized_weight("gate_up_proj", self.gate_up_proj), self._quantized_weight("down_proj", self.down_proj),
@@ -255,8 +261,10 @@ def forward_stage3(experts: nn.Module, gathered_tokens, expert_idxs, experts_per
                            expand_idx=expand_idx)
     if (fuse_permute and expand_idx is None and training.fp8 and expert_idxs.shape[0] > 0
             and isinstance(experts, GptOssExperts)):
+        # the one-node block needs no host-side sizes (see the SwiGLU branch above)
         reverse_shuffle_idxs, grouped_mm_offs, ks, ks_tensor, src_of = group_rows_with_sizes(
-            expert_idxs, experts_per_rank, device=gathered_tokens.device)
+            expert_idxs, experts_per_rank, device=gathered_tokens.device,
+            host_sizes=host_sizes or not experts.one_node(gathered_tokens))
         if experts.bias_fusable(gathered_tokens):
             # both sides: rows gathered by the first quantisation, stored un-permuted (bias added)
             # by the last GEMM; the bias gradients are summed through the same map

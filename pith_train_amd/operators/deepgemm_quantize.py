@@ -50,9 +50,10 @@ def transposed_pitch(m: int) -> int:
     return m + 128 if (m >= 2048 and m % 256 == 0) else m
 
 
-def _empty_transposed(rows: int, m: int, dev) -> torch.Tensor:
-    """``[rows, m]`` FP8 with the row pitch of :func:`transposed_pitch` (a view when padded)."""
-    ld = transposed_pitch(m)
+def _empty_transposed(rows: int, m: int, dev, padded: bool) -> torch.Tensor:
+    """``[rows, m]`` FP8, packed, or (``padded``) with the row pitch of :func:`transposed_pitch`
+    (then a view of a wider buffer when that pitch differs from ``m``)."""
+    ld = transposed_pitch(m) if padded else m
     buf = torch.empty((rows, ld), dtype=FP8, device=dev)
     return buf if ld == m else buf[:, :m]
 
@@ -131,40 +132,43 @@ def fp8cast_rowwise_kmajor(x: torch.Tensor, grouped_mm_offs: torch.Tensor):
     return _rowwise_colwise(x, _lib.PT_CH_KMAJOR, grouped_mm_offs.contiguous())
 
 
-def fp8cast_rowwise_transpose(x: torch.Tensor):
-    """(tok_fp8[M,N], tok_scale[M,ceil(N/128)], t_fp8[N,M], t_scale[N,ceil(M/128)])."""
+def fp8cast_rowwise_transpose(x: torch.Tensor, *, _padded: bool = False):
+    """(tok_fp8[M,N], tok_scale[M,ceil(N/128)], t_fp8[N,M], t_scale[N,ceil(M/128)]), all freshly
+    allocated and contiguous.  ``_padded`` is for this package's dense linear only: ``t_fp8`` may
+    then be a row-padded view (see :func:`transposed_pitch`)."""
     assert x.ndim == 2, f"Expected 2D tensor, got {x.ndim}D"
     x = _prep2d(x)
     M, N = x.shape
     dev = x.device
     out_tok = torch.empty((M, N), dtype=FP8, device=dev)
     scale_tok = torch.empty((M, _cdiv(N, 128)), dtype=torch.float32, device=dev)
-    out_t = _empty_transposed(N, M, dev)
+    out_t = _empty_transposed(N, M, dev, _padded)
     scale_t = torch.empty((N, _cdiv(M, 128)), dtype=torch.float32, device=dev)
     if M and N:
         _lib.call(
             "pt_quant_rowwise_transpose_ld", x.data_ptr(), _lib.dtype_code(x.dtype), M, N,
             x.stride(0) if M > 1 else N, out_tok.data_ptr(), scale_tok.data_ptr(), out_t.data_ptr(),
-            out_t.stride(0) if N > 1 else transposed_pitch(M), scale_t.data_ptr(), _lib.stream_ptr(dev),
+            out_t.stride(0) if N > 1 else M, scale_t.data_ptr(), _lib.stream_ptr(dev),
         )  # fmt: skip
     return out_tok, scale_tok, out_t, scale_t
 
 
-def fp8cast_rowwise_blockwise_transpose(x: torch.Tensor):
-    """(tok_fp8[M,K], tok_scale[M,ceil(K/128)], blk_t_fp8[K,M], blk_t_scale[ceil(K/128),ceil(M/128)])."""
+def fp8cast_rowwise_blockwise_transpose(x: torch.Tensor, *, _padded: bool = False):
+    """(tok_fp8[M,K], tok_scale[M,ceil(K/128)], blk_t_fp8[K,M], blk_t_scale[ceil(K/128),ceil(M/128)]),
+    all freshly allocated and contiguous; ``_padded`` as in :func:`fp8cast_rowwise_transpose`."""
     assert x.ndim == 2, f"Expected 2D tensor, got {x.ndim}D"
     x = _prep2d(x)
     M, K = x.shape
     dev = x.device
     out_tok = torch.empty((M, K), dtype=FP8, device=dev)
     scale_tok = torch.empty((M, _cdiv(K, 128)), dtype=torch.float32, device=dev)
-    out_blk_t = _empty_transposed(K, M, dev)
+    out_blk_t = _empty_transposed(K, M, dev, _padded)
     scale_blk_t = torch.empty((_cdiv(K, 128), _cdiv(M, 128)), dtype=torch.float32, device=dev)
     if M and K:
         _lib.call(
             "pt_quant_rowwise_blockwise_transpose_ld", x.data_ptr(), _lib.dtype_code(x.dtype), M, K,
             x.stride(0) if M > 1 else K, out_tok.data_ptr(), scale_tok.data_ptr(),
-            out_blk_t.data_ptr(), out_blk_t.stride(0) if K > 1 else transposed_pitch(M), scale_blk_t.data_ptr(),
+            out_blk_t.data_ptr(), out_blk_t.stride(0) if K > 1 else M, scale_blk_t.data_ptr(),
             _lib.stream_ptr(dev),
         )  # fmt: skip
     return out_tok, scale_tok, out_blk_t, scale_blk_t

@@ -258,15 +258,18 @@ class FP8ClampedSwiGLUExpertsFunc(torch.autograd.Function):
         assert not scatter_output or row_map is not None, "scatter_output needs the row map"
         if row_map is not None:
             M = row_map.shape[0]
-            x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, row_map)
+            # row_map may be sized for more rows than the routing produced (its tail negative):
+            # every kernel below takes the real row count from grouped_mm_offs on the device
+            x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t_rows(x, row_map, grouped_mm_offs)
         else:
             M = x.shape[0]
             x_fp8, x_s, x_ch_t, x_ch_s = fp8cast_rowwise_colwise_t(x)
+        limit_rows = grouped_mm_offs if row_map is not None else None
         gate_up = torch.empty((M, two_i), device=x.device, dtype=x.dtype)
         m_grouped_fp8_gemm_nt((x_fp8, x_s), (gu_fp8, gu_scale), gate_up, grouped_mm_offs, None,
                               b_gate_up.detach().contiguous())
         del x_fp8, x_s
-        h_fp8, h_s, h_ch_t, h_ch_s = clamped_swiglu_quant(gate_up, alpha, limit)
+        h_fp8, h_s, h_ch_t, h_ch_s = clamped_swiglu_quant(gate_up, alpha, limit, limit_rows)
         out_rows = row_map if scatter_output else None
         out = torch.empty((x.shape[0] if scatter_output else M, H), device=x.device, dtype=x.dtype)
         m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, out_rows,
@@ -292,7 +295,7 @@ class FP8ClampedSwiGLUExpertsFunc(torch.autograd.Function):
         grad_out = grad_out.contiguous()
         out_rows = row_map if scatter_output else None
         if out_rows is not None:
-            dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t_rows(grad_out, out_rows)
+            dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t_rows(grad_out, out_rows, offs)
         else:
             dy_fp8, dy_s, dy_ch_t, dy_ch_s = fp8cast_rowwise_colwise_t(grad_out)
         grad_b_down = _segment_sum_along_rows(grad_out, offs, dn_bias_dtype, out_rows)
@@ -300,7 +303,8 @@ class FP8ClampedSwiGLUExpertsFunc(torch.autograd.Function):
         m_grouped_fp8_dgrad((dy_fp8, dy_s), dn_dg, dn_dg_s, ctx.dn_forward_layout, grad_h, offs)
         schedule_wgrad(w_down, (dy_ch_t, dy_ch_s), (h_ch_t, h_ch_s), offs)
         del dy_fp8, dy_s
-        dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s, col_sum = clamped_swiglu_bwd_quant(grad_h, gate_up, alpha, limit)
+        dgu_fp8, dgu_s, dgu_ch_t, dgu_ch_s, col_sum = clamped_swiglu_bwd_quant(
+            grad_h, gate_up, alpha, limit, offs if row_map is not None else None)
         # groups are whole 128-row tiles: their ends in tiles index the per-tile column sums
         grad_b_gate_up = _segment_sum_along_rows(col_sum, offs // 128, gu_bias_dtype)
         grad_x = torch.empty((rows_x if row_map is not None else M, K), device=grad_out.device, dtype=grad_out.dtype)

@@ -90,7 +90,7 @@ def fp8_act_weight_gemm(input_2d, weight_fp8, scale_weight):
     """y = x @ W.T; returns (output, input_t_fp8[K,M], scale_input_t) - the transposed activation
     is handed back for the later wgrad."""
     m, n = input_2d.shape[0], weight_fp8.shape[0]
-    input_fp8, scale_input, input_t_fp8, scale_input_t = fp8cast_rowwise_blockwise_transpose(input_2d)
+    input_fp8, scale_input, input_t_fp8, scale_input_t = fp8cast_rowwise_blockwise_transpose(input_2d, _padded=True)
     output = _fp8_gemm_nt(
         input_fp8, scale_input, weight_fp8, scale_weight, m, n, input_2d.device, input_2d.dtype
     )
@@ -101,7 +101,7 @@ def fp8_dgrad_wgrad(grad_2d, weight_t_fp8, scale_weight_t, input_t_fp8, scale_in
     """grad_input = grad @ W (through W^T) and weight_grad = grad^T @ x (through x^T), both in
     ``grad_2d``'s dtype."""
     m, n = grad_2d.shape
-    grad_fp8, scale_grad, grad_t_fp8, scale_grad_t = fp8cast_rowwise_transpose(grad_2d)
+    grad_fp8, scale_grad, grad_t_fp8, scale_grad_t = fp8cast_rowwise_transpose(grad_2d, _padded=True)
     grad_input = _fp8_gemm_nt(
         grad_fp8, scale_grad, weight_t_fp8, scale_weight_t, m, k, grad_2d.device, grad_2d.dtype
     )

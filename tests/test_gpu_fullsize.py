@@ -117,8 +117,8 @@ def test_full_size_dense_weight_gradient_split_over_the_reduction_matches_the_si
     for n_out, n_in in ((512, 2048), (4096, 2048)):
         grad = torch.randn((tokens, n_out), generator=g).bfloat16().cuda()
         x = torch.randn((tokens, n_in), generator=g).bfloat16().cuda()
-        _, _, gt, gt_s = DQ.fp8cast_rowwise_transpose(grad)            # grad^T rows, 1x128 scales
-        _, _, xt, xt_s = DQ.fp8cast_rowwise_blockwise_transpose(x)     # x^T, 128x128 scales
+        _, _, gt, gt_s = DQ.fp8cast_rowwise_transpose(grad, _padded=True)            # grad^T rows, 1x128 scales (the dense linear's private row-padded form)
+        _, _, xt, xt_s = DQ.fp8cast_rowwise_blockwise_transpose(x, _padded=True)     # x^T, 128x128 scales
         assert _split_k(n_out, n_in, tokens)[0] > 1
         split = _fp8_gemm_nt(gt, gt_s, xt, xt_s, n_out, n_in, "cuda", torch.float32)
         single = torch.empty((n_out, n_in), device="cuda", dtype=torch.float32)

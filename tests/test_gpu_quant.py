@@ -57,17 +57,24 @@ def test_rowwise_colwise(M, N, dtype):
     _eq(got_t[3], ref[3], "ch_scale")
 
 
-def test_transposed_outputs_of_large_token_counts_are_row_padded_views():
-    """The transposed operands of 2048+ tokens (a multiple of 256) come back as views of buffers
-    with one more 128-byte column per row; the padding is never read as data."""
+def test_transposed_outputs_are_contiguous_as_in_the_reference():
+    """The public quantisers return freshly allocated contiguous tensors whatever the token count
+    (reference: operators/deepgemm_quantize.py:429-482,575-629); only the private form that the
+    dense linear uses pads the rows of the transposed operand, and it holds the same bytes."""
     D = _ops()
-    x = _mk((4096, 256), 5)
-    _, _, t, _ = D.fp8cast_rowwise_transpose(x.cuda())
-    _, _, bt, _ = D.fp8cast_rowwise_blockwise_transpose(x.cuda())
-    for v in (t, bt):
-        assert v.shape == (256, 4096) and v.stride() == (4096 + 128, 1) and not v.is_contiguous()
-    _, _, t2, _ = D.fp8cast_rowwise_transpose(_mk((300, 256), 6).cuda())
-    assert t2.is_contiguous()
+    for shape, seed in (((4096, 256), 5), ((300, 256), 6), ((2048, 384), 7)):
+        x = _mk(shape, seed).cuda()
+        for fn in (D.fp8cast_rowwise_transpose, D.fp8cast_rowwise_blockwise_transpose):
+            got = fn(x)
+            for t in got:
+                assert t.is_contiguous() and t.storage_offset() == 0
+            assert got[2].shape == (shape[1], shape[0]) and got[2].view(-1).numel() == shape[0] * shape[1]
+            padded = fn(x, _padded=True)
+            if shape[0] >= 2048 and shape[0] % 256 == 0:
+                assert padded[2].stride() == (shape[0] + 128, 1)
+            for a, b in zip(got, padded):
+                assert torch.equal(a.view(torch.uint8) if a.dtype != torch.float32 else a,
+                                   b.view(torch.uint8) if b.dtype != torch.float32 else b)
 
 
 def test_rowwise_colwise_all_zero_and_strided():
