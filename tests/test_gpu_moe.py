@@ -8,6 +8,7 @@ tests/test_deepgemm_fp8_linear_correctness.py:14) plus max |err| <= 5e-2 x max |
 2**-4 of the element).
 """
 
+
 import pytest
 import torch
 
@@ -17,15 +18,40 @@ from oracle import moe as OM
 pytestmark = pytest.mark.gpu
 
 
-def _close(got, ref, what, rel=5e-2, diff=1e-3):
+REL = 1e-2  # the stated tolerance: max rel-err <= 1e-2 against the fp32-dequantised reference
+
+
+def _close(got, ref, what, chained=True, diff=1e-3):
+    """calc_diff < 1e-3 always, plus an element bound in one of two regimes.
+
+    chained=False - the tensor is one GEMM away from operands that the oracle and the library
+    quantise from the same bits: every element within REL * |ref| + REL * rms(ref), the bound of the
+    GEMM tests (measured worst case: 0.66 of it).
+
+    chained=True - a quantised operand of the last GEMM was itself computed from GEMM results
+    (h = SwiGLU(gate_up), the activation gradients).  The scaled FP8 MFMA of gfx950 carries about
+    16 significant bits through a 128-deep block (a single GEMM's fp32 result differs from the
+    exact sum of its FP8 products by 1.5e-5 of the rms, measured; every kernel of the library
+    gives the same bits), so a per cent of the bf16 intermediates differ from the oracle's in
+    their last bit, a tenth of those change an e4m3 byte of the re-quantised operand (6-12 % of
+    that element), and an output that sums a few such elements moves by about 1 % of the rms.
+    Asserted: at least 99.5 % of the elements inside the single-GEMM bound (measured: >= 99.88 %)
+    and max |err| <= 4e-2 * max |ref| (measured worst case over all configurations: 2.8e-2)."""
     got, ref = got.detach().float().cpu().double(), ref.double()
     assert got.shape == ref.shape, f"{what}: {tuple(got.shape)} vs {tuple(ref.shape)}"
     assert torch.isfinite(got).all(), what
     d = G.calc_diff(got, ref)
-    worst = (got - ref).abs().max().item()
-    scale = ref.abs().max().item()
     assert d < diff, f"{what}: calc_diff {d:.3e}"
-    assert worst <= rel * scale + 1e-30, f"{what}: max err {worst:.3e} vs max |ref| {scale:.3e}"
+    rms = ref.pow(2).mean().sqrt().item()
+    err = (got - ref).abs()
+    ratio = err / (REL * ref.abs() + REL * rms + 1e-300)
+    if not chained:
+        assert ratio.max().item() <= 1.0, f"{what}: worst element at {ratio.max().item():.3f} x the bound (rms {rms:.3e})"
+        return
+    inside = (ratio <= 1.0).double().mean().item()
+    relmax = (err.max() / ref.abs().max().clamp_min(1e-300)).item()
+    assert inside >= 0.995, f"{what}: only {inside:.4%} of the elements inside the single-GEMM bound"
+    assert relmax <= 4e-2, f"{what}: max |err| = {relmax:.3e} of max |ref|"
 
 
 def _weights(kind, E, H, I, seed):
@@ -261,12 +287,12 @@ def test_fp8_linear_forward_backward(M, K, N, bias):
     y = lin(xc)
     assert y.shape == (2, M // 2, N)
     ref = y_ref if not bias else (y_ref + lin.bias.detach().cpu())
-    _close(y.reshape(M, N), ref, "y")
+    _close(y.reshape(M, N), ref, "y", chained=False)
     y.backward(dy.cuda().view(2, M // 2, N))
-    _close(xc.grad.reshape(M, K), gi_ref, "grad_input")
-    _close(lin.weight.grad, gw_ref, "weight_grad")
+    _close(xc.grad.reshape(M, K), gi_ref, "grad_input", chained=False)
+    _close(lin.weight.grad, gw_ref, "weight_grad", chained=False)
     if bias:
-        _close(lin.bias.grad, dy.float().sum(0), "bias_grad", rel=2e-2)
+        _close(lin.bias.grad, dy.float().sum(0), "bias_grad", chained=False)
 
 
 def test_dense_mlp_and_bf16_switch():
@@ -431,6 +457,25 @@ def test_moe_block_reference_forward_against_the_oracle_chain(family):
         p = getattr(blk.experts, n)
         _close((p if kind == "gpt_oss" else p.weight).grad, bwd[n], f"{family} {n} grad")
     assert xin.grad is not None and torch.isfinite(xin.grad.float()).all() and gate.weight.grad is not None
+    if mlp is None:
+        # The input gradient and the gate's weight gradient against the oracle chain: the experts'
+        # token gradients summed over a token's k copies, plus the path through the routing
+        # weights (combine backward -> gate expression on the selection the kernel made -> logits
+        # GEMM), which is autograd of the reference's expressions on the CPU.
+        from oracle import router as OR
+
+        d_moe2, d_weight, _ = OC.combine_bwd(dy, fwd["out"], topk_weight.cpu())
+        via_experts = bwd["grad_tokens"].view(T, k, H).float().sum(1).bfloat16()
+        xg = x.clone().requires_grad_(True)
+        wg = gate.weight.detach().cpu().clone().requires_grad_(True)
+        if family == "gpt_oss":
+            bg = gate.bias.detach().cpu().clone().requires_grad_(True)
+            _, tw, _ = OR.topk_softmax(torch.nn.functional.linear(xg, wg, bg), k, forced_idx=topk_idx.cpu())
+        else:
+            _, tw, _ = OR.softmax_topk(torch.nn.functional.linear(xg, wg), k, norm_topk_prob=True, forced_idx=topk_idx.cpu())
+        tw.backward(d_weight)
+        _close(xin.grad, (via_experts.float() + xg.grad.float()).bfloat16(), f"{family} input gradient")
+        _close(gate.weight.grad, wg.grad, f"{family} gate weight gradient")
 
 
 def test_moe_combine_without_a_residual_is_the_rounded_weighted_sum():
