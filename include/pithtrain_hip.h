@@ -291,6 +291,9 @@ int pt_group_rows(const int64_t* keys, int64_t m, int32_t num_groups, int32_t al
  * PT_GROUP_ROWS_STATIC_MAX_WORKSPACE (e.g. up to 262144 keys in 256 groups, or 524288 keys in 128).
  * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two
  * threads) race; calls on one stream are ordered and need nothing cleared in between.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress, which may load the
+ * code object) and must be made outside a graph capture; a captured call records that one
+ * address, so two graphs that contain it must not replay at the same time on one GPU either.
  * No counterpart in the reference, which allocates its counters with torch on every call
  * (token_scatter.py:205-207). */
 #define PT_GROUP_ROWS_STATIC_MAX_WORKSPACE ((1 << 20) + 8192)

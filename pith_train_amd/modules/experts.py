@@ -22,7 +22,7 @@ import torch.nn as nn
 from ..dualpipe_utils import FP8WeightCacheControl
 from ..operators import fused_experts
 from ..operators.clamped_swiglu import clamped_swiglu
-from ..operators.deepgemm_quantize import fp8cast_grouped_weight, fp8cast_grouped_weight_cat
+from ..operators.deepgemm_quantize import fp8cast_grouped_weight, fp8cast_grouped_weight_cat, weight_twin_enabled
 from ..operators.grouped_linear import FP8GroupedLinear, FP8GroupedLinearFunc, GroupedLinearFunc
 from ..operators.indexed_bias_add import indexed_bias_add
 from ..operators.silu_mul import silu_mul, silu_mul_halves
@@ -52,7 +52,7 @@ class Qwen3MoeExperts(nn.Module):
         if torch.compiler.is_compiling():
             return fp8cast_grouped_weight_cat(parts)
         ver = FP8WeightCacheControl.version
-        if self._gu_cache is None or self._gu_version != ver:
+        if self._gu_cache is None or self._gu_version != ver or (self._gu_cache[2] is not None) != weight_twin_enabled():
             self._gu_cache = fp8cast_grouped_weight_cat(parts)
             self._gu_version = ver
         return self._gu_cache
@@ -162,7 +162,7 @@ class GptOssExperts(nn.Module):
         if self._wq_version != ver or cache is None:
             cache = self._wq_cache = {}
             self._wq_version = ver
-        if name not in cache:
+        if name not in cache or (cache[name][2] is not None) != weight_twin_enabled():
             cache[name] = fp8cast_grouped_weight(weight)
         return cache[name]
 

@@ -153,8 +153,8 @@ def _forward(ctx, x, gate_up_weights, w_down, grouped_mm_offs, q_gate_up, q_down
     h_fp8, h_s, h_ch_t, h_ch_s = silu_mul_quant(gate_up, grouped_mm_offs if row_map is not None else None)
     out = torch.empty((out_m, H), device=x.device, dtype=x.dtype)
     m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, row_map)
-    gu_dg, gu_dg_s, ctx.gu_forward_layout = dgrad_operand(q_gate_up)
-    dn_dg, dn_dg_s, ctx.dn_forward_layout = dgrad_operand(q_down)
+    gu_dg, gu_dg_s, ctx.gu_forward_layout = dgrad_operand(q_gate_up, gate_up_weights, M)
+    dn_dg, dn_dg_s, ctx.dn_forward_layout = dgrad_operand(q_down, w_down, M)
     ctx.save_for_backward(gu_dg, gu_dg_s, dn_dg, dn_dg_s, grouped_mm_offs, x_ch_t, x_ch_s,
                           gate_up, h_ch_t, h_ch_s, row_map, expand_idx)
     ctx.gate_up_weights, ctx.w_down = gate_up_weights, w_down
@@ -274,8 +274,8 @@ class FP8ClampedSwiGLUExpertsFunc(torch.autograd.Function):
         out = torch.empty((x.shape[0] if scatter_output else M, H), device=x.device, dtype=x.dtype)
         m_grouped_fp8_gemm_nt((h_fp8, h_s), (dn_fp8, dn_scale), out, grouped_mm_offs, out_rows,
                               b_down.detach().contiguous())
-        gu_dg, gu_dg_s, ctx.gu_forward_layout = dgrad_operand(q_gate_up)
-        dn_dg, dn_dg_s, ctx.dn_forward_layout = dgrad_operand(q_down)
+        gu_dg, gu_dg_s, ctx.gu_forward_layout = dgrad_operand(q_gate_up, w_gate_up, M)
+        dn_dg, dn_dg_s, ctx.dn_forward_layout = dgrad_operand(q_down, w_down, M)
         ctx.save_for_backward(gu_dg, gu_dg_s, dn_dg, dn_dg_s, grouped_mm_offs, x_ch_t, x_ch_s,
                               gate_up, h_ch_t, h_ch_s, row_map)
         ctx.weights = (w_gate_up, w_down)

@@ -25,7 +25,10 @@ import torch.nn.functional as F
 from .. import _lib
 from ..dualpipe_utils import FP8WeightCacheControl, WeightGradStore
 from .deepgemm_quantize import (
+    fp8cast_blockwise_transpose_batched,
+    fp8cast_blockwise_transpose_batched_cat,
     fp8cast_grouped_weight,
+    weight_twin_enabled,
     fp8cast_rowwise_colwise_t,
     fp8cast_rowwise_colwise_t_rows,
 )
@@ -258,10 +261,29 @@ def m_grouped_fp8_gemm_nn(a, b, out: torch.Tensor, grouped_mm_offs: torch.Tensor
     return out
 
 
-def dgrad_operand(quantized_weight: tuple):
+# limits of the kernel that reads a weight in its forward layout (32-bit byte offsets, group table)
+_NN_MAX_GRAD_BYTES = 2**31
+_NN_MAX_OUT_BYTES = 2**32
+_NN_MAX_GROUPS = 2048
+
+
+def dgrad_operand(quantized_weight: tuple, weight=None, rows: int = 0):
     """(fp8, scale, forward_layout) of the weight operand the input-gradient GEMM reads: the
-    transposed twin when the tuple has one, else the forward-layout tensors themselves."""
+    transposed twin when the tuple has one, else the forward-layout tensors themselves.
+
+    The kernel that reads the forward layout addresses its operands through 32-bit byte offsets:
+    the quantised gradient ``[rows, out_features]`` must stay below 2 GiB and the result
+    ``[rows, in_features]`` (2 bytes per element) below 4 GiB.  Past that (``rows`` and the bf16
+    ``weight``, or the tuple of weights whose rows the quantised operand concatenates, are given by
+    the forward for this check) the twin is built here, once, instead of failing in the backward."""
     w_fp8, w_scale, w_t_fp8, w_t_scale = quantized_weight
+    if w_t_fp8 is None and weight is not None:
+        n_out, n_in = w_fp8.shape[1], w_fp8.shape[2]
+        if rows * n_out >= _NN_MAX_GRAD_BYTES or rows * n_in * 2 >= _NN_MAX_OUT_BYTES or w_fp8.shape[0] > _NN_MAX_GROUPS:
+            if isinstance(weight, (tuple, list)):
+                _, _, w_t_fp8, w_t_scale = fp8cast_blockwise_transpose_batched_cat([p_.detach() for p_ in weight])
+            else:
+                _, _, w_t_fp8, w_t_scale = fp8cast_blockwise_transpose_batched(weight)
     if w_t_fp8 is None:
         return w_fp8, w_scale, True
     return w_t_fp8, w_t_scale, False
@@ -324,7 +346,7 @@ class FP8GroupedLinearFunc(torch.autograd.Function):
             bias.detach().contiguous() if bias is not None else None,
         )
         ctx.bias_dtype = bias.dtype if bias is not None else None
-        dg_fp8, dg_scale, ctx.dgrad_forward_layout = dgrad_operand(quantized_weight)
+        dg_fp8, dg_scale, ctx.dgrad_forward_layout = dgrad_operand(quantized_weight, weight, M)
         ctx.save_for_backward(
             dg_fp8, dg_scale, grouped_mm_offs, input_ch_t, scale_input_ch, ks_tensor,
             in_rows, out_rows,
@@ -378,8 +400,10 @@ class FP8GroupedLinear(nn.Module):
         if torch.compiler.is_compiling():
             return fp8cast_grouped_weight(self.weight)
         ver = FP8WeightCacheControl.version
-        if self._wq_version == ver and self._wq_cache is not None:
-            return self._wq_cache
+        cache = self._wq_cache
+        # a cached tuple is reused only in the shape the twin switch asks for now
+        if self._wq_version == ver and cache is not None and (cache[2] is not None) == weight_twin_enabled():
+            return cache
         result = fp8cast_grouped_weight(self.weight)
         self._wq_cache = result
         self._wq_version = ver

@@ -166,13 +166,22 @@ def _define_ops(namespace: str):
 
 
 _fp8_linear_fwd, _fp8_linear_bwd = _define_ops("pith_train_amd")
+# The reference registers the same two ops as pithtrain::fp8_linear_fwd / fp8_linear_bwd; code that
+# finds them by qualified name (torch.ops.pithtrain.*) gets these kernels when this module is
+# imported first.  When the reference's own module was imported first the names are taken and stay
+# the reference's; importing the reference's module after this one fails in its own registration.
+# PITHTRAIN_OPS_OWNER says which of the two happened ("pith_train_amd" or "other").
 try:
-    # The reference registers the same two ops as pithtrain::fp8_linear_fwd / fp8_linear_bwd; code
-    # that finds them by qualified name (torch.ops.pithtrain.*) gets these kernels.  When the
-    # reference's own module was imported first the names are taken and stay the reference's.
     _define_ops("pithtrain")
-except RuntimeError:
-    pass
+    PITHTRAIN_OPS_OWNER = "pith_train_amd"
+except RuntimeError as exc:
+    import warnings
+
+    PITHTRAIN_OPS_OWNER = "other"
+    warnings.warn(
+        "pithtrain::fp8_linear_fwd / fp8_linear_bwd were registered before pith_train_amd was imported "
+        f"and keep their first implementation ({exc}); FP8Linear of this package is unaffected "
+        "(it calls pith_train_amd::fp8_linear_*)", RuntimeWarning, stacklevel=2)
 
 
 class FP8Linear(nn.Linear):

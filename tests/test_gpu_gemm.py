@@ -255,6 +255,38 @@ def test_m_grouped_nn_reads_the_forward_layout_weight_with_the_bits_of_nt(sizes,
         assert (out_s.cpu()[untouched] == 7.0).all()
 
 
+@pytest.mark.parametrize("sizes", [[256], [256, 384]])
+def test_m_grouped_nn_reads_nothing_past_a_ragged_reduction(sizes):
+    """The reduction-major b operand of a ragged reduction (K = 400: 16 rows into the last
+    128-block) lies inside a larger buffer whose every other byte is 0xFF, an e4m3 NaN: the rows of
+    a reduction block past a group's K rows belong to the next group or to that padding, and the
+    loader leaves them to the range check of the group's buffer descriptor.  A byte read from
+    there would meet a zero of the a operand and give NaN; the result must be finite and equal to
+    the NT form's bit for bit."""
+    from pith_train_amd.operators.grouped_linear import m_grouped_fp8_gemm_nn, m_grouped_fp8_gemm_nt
+
+    N, K = 272, 400
+    ks, offs = _groups(sizes)
+    M, Gn = int(offs[-1]), len(sizes)
+    x = _rand((M, K), 71)
+    w = _rand((Gn, N, K), 73, 0.02)
+    a, sa, _, _ = Q.fp8cast_rowwise_colwise(x)
+    b, sb, _, _ = Q.fp8cast_blockwise_transpose_batched(w)
+    big = torch.full((Gn * K * N + 256 * N,), 0xFF, dtype=torch.uint8, device="cuda")
+    bt = big[: Gn * K * N].view(Gn, K, N)
+    bt.copy_(b.transpose(1, 2).contiguous().view(torch.uint8).cuda())
+    bt = bt.view(torch.float8_e4m3fn)
+    sbt = sb.transpose(1, 2).contiguous().cuda()
+    out_nn = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    out_nt = out_nn.clone()
+    m_grouped_fp8_gemm_nn((a.cuda(), sa.cuda()), (bt, sbt), out_nn, offs.cuda())
+    m_grouped_fp8_gemm_nt((a.cuda(), sa.cuda()), (b.cuda(), sb.cuda()), out_nt, offs.cuda())
+    rows = int(offs[-1])
+    assert torch.isfinite(out_nn[:rows].float()).all(), "a byte past the group's reduction rows was read"
+    assert torch.equal(out_nn[:rows], out_nt[:rows])
+    assert (big[Gn * K * N :] == 0xFF).all()
+
+
 def test_m_grouped_nt_with_more_tiles_per_workgroup_than_the_tile_table_holds(gemm_kernel):
     """Four groups of 25600 rows x 8192 columns: 12800 tiles, 50 per workgroup, so the grouped
     tile decode (group search, row tile inside the group) also runs on the fly for the last tiles.

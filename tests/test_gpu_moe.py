@@ -478,6 +478,47 @@ def test_moe_block_reference_forward_against_the_oracle_chain(family):
         _close(gate.weight.grad, wg.grad, f"{family} gate weight gradient")
 
 
+@pytest.mark.parametrize("kind", ["fused", "split", "gpt_oss"])
+def test_stage3_builds_the_weight_twin_when_the_forward_layout_kernel_cannot_address_the_problem(kind, monkeypatch):
+    """The input-gradient kernel on forward-layout weights has 32-bit limits; past them the forward
+    builds the transposed twin and the backward takes the NT form.  With the limits lowered to
+    nothing the results are the default path's, bit for bit."""
+    from pith_train_amd.dualpipe_utils import FP8WeightCacheControl
+    from pith_train_amd.modules.experts import forward_stage3
+    from pith_train_amd.operators import grouped_linear as GL
+
+    E, H, I, T, k = 8, 256, 384, 700, 2
+    ids = OM.make_routing(T, E, k, seed=5).reshape(-1).cuda()
+    w = _weights(kind, E, H, I, 6)
+    g = torch.Generator().manual_seed(7)
+    x0 = torch.randn((T * k, H), generator=g).bfloat16().cuda()
+    dy = torch.randn((T * k, H), generator=g).bfloat16().cuda()
+    calls = []
+    real = GL.m_grouped_fp8_gemm_nn
+
+    def counting(*a, **kw):
+        calls.append(1)
+        return real(*a, **kw)
+
+    monkeypatch.setattr(GL, "m_grouped_fp8_gemm_nn", counting)
+
+    def run():
+        mod, params = _build(kind, E, H, I, w)
+        FP8WeightCacheControl.step()
+        x = x0.clone().requires_grad_(True)
+        out = forward_stage3(mod, x, ids, E)
+        out.backward(dy)
+        return [out.detach(), x.grad] + [p.grad for p in params.values()]
+
+    a = run()
+    assert calls, "the default path reads the forward-layout weights"
+    calls.clear()
+    monkeypatch.setattr(GL, "_NN_MAX_GRAD_BYTES", 1)
+    b = run()
+    assert not calls, "past the limit the twin is built and the NT form runs"
+    assert len(a) == len(b) and all(torch.equal(u, v) for u, v in zip(a, b))
+
+
 def test_moe_combine_without_a_residual_is_the_rounded_weighted_sum():
     from oracle import combine as OC
     from pith_train_amd.operators.moe_combine import moe_combine
