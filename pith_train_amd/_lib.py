@@ -13,7 +13,8 @@ from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libpithtrain_hip.so")
+# PITHTRAIN_HIP_LIB: another build of the library (measurement builds, see csrc/Makefile)
+LIB_PATH = os.environ.get("PITHTRAIN_HIP_LIB") or os.path.join(_HERE, "libpithtrain_hip.so")
 
 PT_BF16, PT_F32, PT_F16 = 0, 1, 2
 PT_CH_ROWMAJOR, PT_CH_TRANSPOSED, PT_CH_KMAJOR = 0, 1, 2

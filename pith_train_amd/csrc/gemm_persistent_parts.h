@@ -15,6 +15,11 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 static constexpr int kMaxGroupsGemm = 2048;
+#ifdef PT_GEMM_ABLATE_STORES
+static constexpr bool kAblateStores = true;
+#else
+static constexpr bool kAblateStores = false;
+#endif
 static constexpr uint32_t kOob = 0x80000000u;  // per-lane offset that is out of range for every descriptor used here
 static constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
 
@@ -377,15 +382,17 @@ __device__ __forceinline__ void store_tile(v16f (&acc)[TM][TN], const GemmArgs& 
   const bool wide_ok = p.out_dtype != PT_F32 && (p.ldo & 7) == 0 && (((uintptr_t)p.out) & 15) == 0 &&
                        (MODE != GEMM_K_GROUPED || (p.out_stride_g & 7) == 0);
   // The descriptor ends after the tile's last valid row: stores to ragged rows are dropped.
+  // (PT_GEMM_ABLATE_STORES, measurement builds only: it ends before the first, so every store
+  // instruction runs and nothing is written.)
   char* outp = (char*)p.out + (MODE == GEMM_K_GROUPED ? (int64_t)T.g * p.out_stride_g * esz : 0);
-  const __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(outp, 0, (int)((uint32_t)T.a_lim * pitch), kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t rs_out = __builtin_amdgcn_make_buffer_rsrc(outp, 0, kAblateStores ? 0 : (int)((uint32_t)T.a_lim * pitch), kRsrcFlags);
   const uint32_t s_tile = (uint32_t)(T.a_row0 + wm0) * pitch + (uint32_t)(T.b_row0 + wn0) * esz;
   const int colw = T.b_row0 + wn0 + (lane & 31);
   static_assert(TN % 2 == 0, "the wide stores take column blocks in pairs");
   if (MODE == GEMM_M_GROUPED && p.out_row_index) {
     // Result row r goes to output row out_row_index[r] (the un-permute folded into the store);
     // rows of the group's padding map to a negative index and are dropped.
-    const __amdgpu_buffer_rsrc_t rs_sc = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, (int)((uint32_t)p.out_rows * pitch), kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs_sc = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, kAblateStores ? 0 : (int)((uint32_t)p.out_rows * pitch), kRsrcFlags);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       // one index load for the block row (lane -> row lane%32), handed to the lanes that store the row

@@ -26,6 +26,18 @@
 #include "gemm_persistent_parts.h"
 #include <type_traits>
 
+// Measurement builds only (never defined by the Makefile's default target): parts of the main loop
+// compiled out to see what the rest costs.  PT_GEMM_ABLATE_MFMA: no MFMAs (the fragment reads go
+// with them, nothing consumes their results).  PT_GEMM_ABLATE_LOADS: 1 = every operand and scale
+// load is issued out of range (the instruction runs, nothing is fetched), 2 = not issued at all.
+// The results of such builds are garbage; only their timing means something.
+#ifndef PT_GEMM_ABLATE_MFMA
+#define PT_GEMM_ABLATE_MFMA 0
+#endif
+#ifndef PT_GEMM_ABLATE_LOADS
+#define PT_GEMM_ABLATE_LOADS 0
+#endif
+
 namespace pt {
 
 // BT: the b operand is given reduction-major, [red][rows_b] with row pitch ldb (the forward layout of
@@ -208,6 +220,8 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
   // Load number k (0 <= k < NP) of the step set up by issue_begin.  The wave-load numbers keep the
   // parity of the wave (the LDS swizzle of a load depends on it, see above).
   auto issue_piece = [&](int k) {
+    if (PT_GEMM_ABLATE_LOADS == 2) return;
+    if (PT_GEMM_ABLATE_LOADS == 1) { l_in = false; l_ok = false; }
     if (k < 2) {
       const int q = 16 * k + 8 * l_half + wave;
       dma16(rs_a, (l_in && 8 * q < l_a_rows) ? va : kOob, l_soA + (uint32_t)(8 * q) * (uint32_t)p.lda, l_sA + q * 1024);
@@ -343,7 +357,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
       for (int m = 0; m < 8; ++m) {
         const int i = m & 1, j = (m >> 1) & 1, ks = m >> 2;
         const int late = BT ? ks : j, early = BT ? j : ks;
-        if (wave_active) mfma_sel<false>(fa[2 * ks + i], fb[late][early], acc[i][j], i, sca, j, scb);
+        if (wave_active && !PT_GEMM_ABLATE_MFMA) mfma_sel<false>(fa[2 * ks + i], fb[late][early], acc[i][j], i, sca, j, scb);
 #pragma unroll
         for (int k = m * NP / 8; k < (m + 1) * NP / 8; ++k) issue_piece(k);
         if (m == 0) fb[1][0] = read_b(gs, 1, 0);
@@ -361,7 +375,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
       for (int m = 0; m < 8; ++m) {
         const int i = m & 1, j = (m >> 1) & 1, ks = m >> 2;
         const int late = BT ? ks : j, early = BT ? j : ks;
-        if (wave_active) mfma_sel<false>(fa[2 * ks + i], fb[late][early], acc[2 + i][j], 2 + i, sca, j, scb);
+        if (wave_active && !PT_GEMM_ABLATE_MFMA) mfma_sel<false>(fa[2 * ks + i], fb[late][early], acc[2 + i][j], 2 + i, sca, j, scb);
 #pragma unroll
         for (int k = m * NP / 8; k < (m + 1) * NP / 8; ++k) issue_piece(k);
         if (m == 0) read_scales(gs + 1, sca_n, scb_n);

@@ -1,0 +1,44 @@
+// Probe of the write path on gfx950 (not part of the library): how the rate at which compute
+// units can write result tiles depends on how many XCDs and how many CUs per XCD write at once.
+// One workgroup per CU (256 launched; workgroup b runs on XCD b % 8), eight waves each, every
+// wave-store writes 8 rows x 128 bytes (the shape of the GEMM's result stores: 16 bytes per lane,
+// row pitch 4096 bytes).  Active workgroups write 4 MiB each, the others return at once.
+// Prints GB/s per active CU and in total.
+// Build: hipcc -O3 --offload-arch=gfx950 store_path.hip -o store_path
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <stdint.h>
+typedef int v4i __attribute__((ext_vector_type(4)));
+#define CHECK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("%s: %s\n", #x, hipGetErrorString(e)); exit(1); } } while (0)
+
+__global__ __launch_bounds__(512, 1) void store_kernel(uint8_t* buf, int xcds, int cus_per_xcd, int reps) {
+  if ((int)(blockIdx.x & 7) >= xcds || (int)(blockIdx.x >> 3) >= cus_per_xcd) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint8_t* base = buf + (size_t)blockIdx.x * (4u << 20);
+  const uint32_t pitch = 4096;  // 1024 rows x 4096 bytes = 4 MiB per workgroup
+  const v4i val = v4i{lane, wave, 3, 4};
+  for (int r = 0; r < reps; ++r)
+    for (int q = wave; q < 128 * 32; q += 8) {  // 128 row groups of 8 rows x 32 column chunks of 128 bytes
+      const int rg = q & 127, c = q >> 7;
+      *(v4i*)(base + (size_t)(rg * 8 + (lane >> 3)) * pitch + c * 128 + (lane & 7) * 16) = val;
+    }
+}
+
+int main() {
+  uint8_t* buf; CHECK(hipMalloc(&buf, (size_t)1 << 30));
+  hipEvent_t a, b; CHECK(hipEventCreate(&a)); CHECK(hipEventCreate(&b));
+  for (int xcds : {1, 2, 4, 8})
+    for (int cus : {1, 4, 8, 16, 32}) {
+      const int reps = 4;
+      store_kernel<<<256, 512>>>(buf, xcds, cus, 1);
+      CHECK(hipEventRecord(a));
+      store_kernel<<<256, 512>>>(buf, xcds, cus, reps);
+      CHECK(hipEventRecord(b)); CHECK(hipEventSynchronize(b));
+      float ms; CHECK(hipEventElapsedTime(&ms, a, b));
+      const double bytes = (double)xcds * cus * reps * (4u << 20);
+      printf("XCDs %d x CUs %2d: %6.1f GB/s per CU, %5.2f TB/s in total\n", xcds, cus, bytes / (ms * 1e-3) / 1e9 / (xcds * cus), bytes / (ms * 1e-3) / 1e12);
+      fflush(stdout);
+    }
+  return 0;
+}
