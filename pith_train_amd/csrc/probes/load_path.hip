@@ -41,8 +41,10 @@ __global__ __launch_bounds__(512, 1) void stream_kernel(const uint8_t* buf, uint
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
   // shared: all workgroups of an XCD (blockIdx & 7) read the same region
   // shared == 2: every workgroup walks its own 4 MiB of the buffer once (HBM-resident data)
-  const uint8_t* base = buf + (size_t)(shared == 1 ? (blockIdx.x & 7) : blockIdx.x) * (shared == 2 ? (4u << 20) : region);
+  // shared == 3: up to four workgroups walk 128 MiB each, starting 256 MiB into the buffer (never touched before)
+  const uint8_t* base = buf + (size_t)(shared == 1 ? (blockIdx.x & 7) : blockIdx.x) * (shared == 2 ? (4u << 20) : shared == 3 ? (128u << 20) : region);
   if (shared == 2) region = 4u << 20;
+  if (shared == 3) { region = 128u << 20; base += (size_t)256 << 20; }
   const v4i rs = make_rsrc(base, region);
   const uint32_t voff = (uint32_t)(lane >> 3) * pitch + (lane & 7) * 16;
   const uint32_t rows = region / pitch, cols = pitch / 128, row_groups = rows / 8;
@@ -75,7 +77,7 @@ template <int D, int MODE>
 static double run(const uint8_t* buf, uint32_t region, uint32_t pitch, int iters, int blocks, int shared) {
   CHECK(hipFuncSetAttribute((const void*)stream_kernel<D, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
   hipEvent_t a, b; CHECK(hipEventCreate(&a)); CHECK(hipEventCreate(&b));
-  stream_kernel<D, MODE><<<blocks, 512, 128 * 1024>>>(buf, region, pitch, iters / 4 + 1, shared, nullptr);
+  if (shared != 3) stream_kernel<D, MODE><<<blocks, 512, 128 * 1024>>>(buf, region, pitch, iters / 4 + 1, shared, nullptr);
   CHECK(hipEventRecord(a));
   stream_kernel<D, MODE><<<blocks, 512, 128 * 1024>>>(buf, region, pitch, iters, shared, nullptr);
   CHECK(hipEventRecord(b)); CHECK(hipEventSynchronize(b));
@@ -95,5 +97,13 @@ int main() {
 #define RUN(D, MODE) { const int iters = tgt / (8 * D * 1024); double g = run<D, MODE>(buf, region, pitch, iters, blocks, shared); printf("   %-28s D=%2d: %6.1f GB/s per CU, %5.2f TB/s\n", names[MODE], D, g, g * blocks / 1e3); fflush(stdout); }
       RUN(4, 0) RUN(8, 0) RUN(16, 0) RUN(4, 1) RUN(8, 1) RUN(16, 1) RUN(4, 2) RUN(16, 3)
     }
+  // cold data: nothing of these regions is in any cache (the buffer was written once, long ago, and is four times the
+  // memory-side cache); every variant walks the same region, so all but the first may find it in the memory-side cache
+  for (int blocks : {1, 4}) {
+    printf("blocks %3d, 128 MiB per workgroup walked once (cold):\n", blocks);
+    const int shared = 3;
+    const int tgt = 128 << 20;
+    RUN(16, 1) RUN(16, 0) RUN(4, 1) RUN(1, 1)
+  }
   return 0;
 }
