@@ -12,14 +12,15 @@
 typedef int v4i __attribute__((ext_vector_type(4)));
 #define CHECK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("%s: %s\n", #x, hipGetErrorString(e)); exit(1); } } while (0)
 
-__global__ __launch_bounds__(512, 1) void store_kernel(uint8_t* buf, int xcds, int cus_per_xcd, int reps) {
+__global__ __launch_bounds__(512, 1) void store_kernel(uint8_t* buf, int xcds, int cus_per_xcd, int reps, int waves) {
   if ((int)(blockIdx.x & 7) >= xcds || (int)(blockIdx.x >> 3) >= cus_per_xcd) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (wave >= waves) return;
   uint8_t* base = buf + (size_t)blockIdx.x * (4u << 20);
   const uint32_t pitch = 4096;  // 1024 rows x 4096 bytes = 4 MiB per workgroup
   const v4i val = v4i{lane, wave, 3, 4};
   for (int r = 0; r < reps; ++r)
-    for (int q = wave; q < 128 * 32; q += 8) {  // 128 row groups of 8 rows x 32 column chunks of 128 bytes
+    for (int q = wave; q < 128 * 32; q += waves) {  // 128 row groups of 8 rows x 32 column chunks of 128 bytes
       const int rg = q & 127, c = q >> 7;
       *(v4i*)(base + (size_t)(rg * 8 + (lane >> 3)) * pitch + c * 128 + (lane & 7) * 16) = val;
     }
@@ -31,14 +32,25 @@ int main() {
   for (int xcds : {1, 2, 4, 8})
     for (int cus : {1, 4, 8, 16, 32}) {
       const int reps = 4;
-      store_kernel<<<256, 512>>>(buf, xcds, cus, 1);
+      store_kernel<<<256, 512>>>(buf, xcds, cus, 1, 8);
       CHECK(hipEventRecord(a));
-      store_kernel<<<256, 512>>>(buf, xcds, cus, reps);
+      store_kernel<<<256, 512>>>(buf, xcds, cus, reps, 8);
       CHECK(hipEventRecord(b)); CHECK(hipEventSynchronize(b));
       float ms; CHECK(hipEventElapsedTime(&ms, a, b));
       const double bytes = (double)xcds * cus * reps * (4u << 20);
       printf("XCDs %d x CUs %2d: %6.1f GB/s per CU, %5.2f TB/s in total\n", xcds, cus, bytes / (ms * 1e-3) / 1e9 / (xcds * cus), bytes / (ms * 1e-3) / 1e12);
       fflush(stdout);
     }
+  // all 256 CUs, fewer waves of each writing (the same bytes per CU)
+  for (int waves : {1, 2, 4, 8}) {
+    const int reps = 4;
+    store_kernel<<<256, 512>>>(buf, 8, 32, 1, waves);
+    CHECK(hipEventRecord(a));
+    store_kernel<<<256, 512>>>(buf, 8, 32, reps, waves);
+    CHECK(hipEventRecord(b)); CHECK(hipEventSynchronize(b));
+    float ms; CHECK(hipEventElapsedTime(&ms, a, b));
+    const double bytes = 256.0 * reps * (4u << 20);
+    printf("256 CUs, %d writing wave(s) each: %6.1f GB/s per CU, %5.2f TB/s in total\n", waves, bytes / (ms * 1e-3) / 1e9 / 256, bytes / (ms * 1e-3) / 1e12);
+  }
   return 0;
 }
