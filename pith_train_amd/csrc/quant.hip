@@ -11,7 +11,46 @@
 #include "common.h"
 #include <type_traits>
 
+// Cache policy of the streaming accesses (bits; the default is what measured best inside the
+// training step, the others are measurement builds: make EXTRA=-DPT_QUANT_NT=<bits>):
+//   1  non-temporal loads in the weight kernels (128x128-scaled)     4  their stores
+//   2  non-temporal loads in the activation kernels (row-scaled)      8  their stores
+//   16 non-temporal stores of the activation kernels' transposed twin only
+//   32 non-temporal loads in the fused SwiGLU prologues
+// Weights are read once per step and their FP8 form (0.6 GB for a 128-expert layer) is larger
+// than the memory-side cache, so keeping either in the caches only evicts what the next GEMM
+// needs: 1 + 4 take 1.5 % off the Qwen3-30B-A3B step.  gate_up and grad_h are read once by the
+// SwiGLU prologues: 32 takes another 0.6 %.  Activation outputs are the next GEMM's operands and
+// want to stay in the memory-side cache: 8 or 16 make the step 0.5-2 % slower although the
+// kernels themselves, timed alone back to back, get up to 24 % faster.
+#ifndef PT_QUANT_NT
+#define PT_QUANT_NT (1 + 4 + 32)
+#endif
+
 namespace pt {
+
+typedef uint32_t q_u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t q_u2 __attribute__((ext_vector_type(2)));
+template <bool W> __device__ __forceinline__ uint4 q_load16(const void* p) {
+  if (PT_QUANT_NT & (W ? 1 : 2)) { const q_u4 v = __builtin_nontemporal_load(reinterpret_cast<const q_u4*>(p)); return make_uint4(v.x, v.y, v.z, v.w); }
+  return *reinterpret_cast<const uint4*>(p);
+}
+// the loads of the fused SwiGLU prologues (bit 32)
+__device__ __forceinline__ void q_load8_pro(const void* p, float* v) {
+  uint4 u;
+  if (PT_QUANT_NT & 32) { const q_u4 t = __builtin_nontemporal_load(reinterpret_cast<const q_u4*>(p)); u = make_uint4(t.x, t.y, t.z, t.w); }
+  else u = *reinterpret_cast<const uint4*>(p);
+  v[0] = bf16_lo(u.x); v[1] = bf16_hi(u.x); v[2] = bf16_lo(u.y); v[3] = bf16_hi(u.y);
+  v[4] = bf16_lo(u.z); v[5] = bf16_hi(u.z); v[6] = bf16_lo(u.w); v[7] = bf16_hi(u.w);
+}
+template <bool W> __device__ __forceinline__ void q_store8(void* p, uint32_t lo, uint32_t hi) {
+  if (PT_QUANT_NT & (W ? 4 : 8)) { __builtin_nontemporal_store(q_u2{lo, hi}, reinterpret_cast<q_u2*>(p)); return; }
+  *reinterpret_cast<uint2*>(p) = make_uint2(lo, hi);
+}
+template <bool W> __device__ __forceinline__ void q_store16(void* p, uint4 v) {  // the transposed twin
+  if (PT_QUANT_NT & (W ? 4 : 8 + 16)) { __builtin_nontemporal_store(q_u4{v.x, v.y, v.z, v.w}, reinterpret_cast<q_u4*>(p)); return; }
+  *reinterpret_cast<uint4*>(p) = v;
+}
 
 enum { A_ROW = 0, A_BLOCK = 1 };                       // scaling of the same-orientation output
 enum { B_COL = 0, B_BLOCK = 1 };                       // scaling of the twin
@@ -84,8 +123,8 @@ template <> struct Loader<float> {
 template <typename T> struct Frag;
 template <> struct Frag<bf16_tag> {
   uint32_t w[8][4];
-  __device__ __forceinline__ void load_row(int i, const void* p) {
-    const uint4 u = *reinterpret_cast<const uint4*>(p);
+  template <bool W = false> __device__ __forceinline__ void load_row(int i, const void* p) {
+    const uint4 u = q_load16<W>(p);
     w[i][0] = u.x; w[i][1] = u.y; w[i][2] = u.z; w[i][3] = u.w;
   }
   __device__ __forceinline__ void zero_row(int i) { w[i][0] = w[i][1] = w[i][2] = w[i][3] = 0u; }
@@ -109,7 +148,7 @@ template <> struct Frag<bf16_tag> {
 // the half-to-float conversion; none of the packed-bf16 shortcuts apply.
 template <> struct Frag<f16_tag> {
   uint32_t w[8][4];
-  __device__ __forceinline__ void load_row(int i, const void* p) {
+  template <bool W = false> __device__ __forceinline__ void load_row(int i, const void* p) {
     const uint4 u = *reinterpret_cast<const uint4*>(p);
     w[i][0] = u.x; w[i][1] = u.y; w[i][2] = u.z; w[i][3] = u.w;
   }
@@ -132,7 +171,7 @@ template <> struct Frag<f16_tag> {
 };
 template <> struct Frag<float> {
   float v[8][8];
-  __device__ __forceinline__ void load_row(int i, const void* p) { Loader<float>::load8(p, v[i]); }
+  template <bool W = false> __device__ __forceinline__ void load_row(int i, const void* p) { Loader<float>::load8(p, v[i]); }
   __device__ __forceinline__ void zero_row(int i) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[i][j] = 0.f;
@@ -203,10 +242,10 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
       if (FULL || (col_ok && row0 + i < p.M)) {
         const int64_t r = row0 + i + gate[i & 1];
         float d[8], g[8], u[8], dg[8], du[8];
-        st_bf16::load8(xb + (r * p.ldx + col0) * 2, d);
+        q_load8_pro(xb + (r * p.ldx + col0) * 2, d);
         const char* gp = (const char*)p.x2 + (r * p.ldx2 + col0) * 2;
-        st_bf16::load8(gp, g);
-        st_bf16::load8(gp + p.half * 2, u);
+        q_load8_pro(gp, g);
+        q_load8_pro(gp + p.half * 2, u);
 #pragma unroll
         for (int j = 0; j < 8; ++j) silu_mul_b(d[j], g[j], u[j], dg[j], du[j]);
         f.w[i][0] = pack_bf16x2(dg[0], dg[1]); f.w[i][1] = pack_bf16x2(dg[2], dg[3]);
@@ -230,8 +269,8 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
       if (FULL || (col_ok && row0 + i < p.M)) {
         const char* gp = xb + ((row0 + i) * p.ldx + 2 * col0) * 2;
         float a[8], b[8], o[8];
-        st_bf16::load8(gp, a);
-        st_bf16::load8(gp + 16, b);
+        q_load8_pro(gp, a);
+        q_load8_pro(gp + 16, b);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           o[j] = cswiglu_f(a[2 * j], a[2 * j + 1], p.alpha, p.limit);
@@ -254,7 +293,7 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
         const uint2 dw = *reinterpret_cast<const uint2*>(xb + (r * p.ldx + (col0 >> 1)) * 2);
         const float d[4] = {bf16_lo(dw.x), bf16_hi(dw.x), bf16_lo(dw.y), bf16_hi(dw.y)};
         float a[8], o[8];
-        st_bf16::load8((const char*)p.x2 + (r * p.ldx2 + col0) * 2, a);
+        q_load8_pro((const char*)p.x2 + (r * p.ldx2 + col0) * 2, a);
 #pragma unroll
         for (int j = 0; j < 4; ++j) cswiglu_b(d[j], a[2 * j], a[2 * j + 1], p.alpha, p.limit, o[2 * j], o[2 * j + 1]);
         f.w[i][0] = pack_bf16x2(o[0], o[1]); f.w[i][1] = pack_bf16x2(o[2], o[3]);
@@ -275,18 +314,18 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
         float g[8], u[8], o[8];
         if (PRO == PRO_SILU_FWD) {
           const char* gp = xb + (r * p.ldx + col0) * 2;
-          st_bf16::load8(gp, g);
-          st_bf16::load8(gp + p.half * 2, u);
+          q_load8_pro(gp, g);
+          q_load8_pro(gp + p.half * 2, u);
 #pragma unroll
           for (int j = 0; j < 8; ++j) o[j] = silu_mul_f(g[j], u[j]);
         } else {
           const bool up_half = col0 >= p.half;
           const int64_t cc = col0 - (up_half ? p.half : 0);
           float d[8];
-          st_bf16::load8(xb + (r * p.ldx + cc) * 2, d);
+          q_load8_pro(xb + (r * p.ldx + cc) * 2, d);
           const char* gp = (const char*)p.x2 + (r * p.ldx2 + cc) * 2;
-          st_bf16::load8(gp, g);
-          st_bf16::load8(gp + p.half * 2, u);
+          q_load8_pro(gp, g);
+          q_load8_pro(gp + p.half * 2, u);
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             float dg, du;
@@ -320,7 +359,7 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
       const char* base = xb + (row0 * p.ldx + col0) * Loader<T>::kBytes;
       const int64_t pitch = p.ldx * Loader<T>::kBytes;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) f.load_row(i, base + i * pitch);
+      for (int i = 0; i < 8; ++i) f.template load_row<AM == A_BLOCK>(i, base + i * pitch);
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -390,7 +429,7 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
       if (FULL || row0 + i < p.M) {
         uint8_t* dst = ab + (row0 + i) * p.N + col0;
         if (FULL || p.vec_out) {
-          if (FULL || col0 < p.N) *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+          if (FULL || col0 < p.N) q_store8<AM == A_BLOCK>(dst, lo, hi);
         } else {
 #pragma unroll
           for (int j = 0; j < 8; ++j)
@@ -529,7 +568,7 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
       if (FULL || row0 + i < p.M) {
         uint8_t* dst = bb + (row0 + i) * p.N + col0;
         if (FULL || p.vec_out) {
-          if (FULL || col0 < p.N) *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+          if (FULL || col0 < p.N) q_store8<AM == A_BLOCK>(dst, lo, hi);
         } else {
 #pragma unroll
           for (int j = 0; j < 8; ++j)
@@ -603,7 +642,7 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
       const uint4 val = *reinterpret_cast<const uint4*>(&s_t[n * 128 + ((mc ^ ((n >> 3) & 7)) * 16)]);
       uint8_t* dst = base + n * ld + mc * 16;
       if (FULL || p.vec_out_t) {
-        if (FULL || gm < p.M) *reinterpret_cast<uint4*>(dst) = val;
+        if (FULL || gm < p.M) q_store16<AM == A_BLOCK>(dst, val);
       } else {
         const uint32_t w[4] = {val.x, val.y, val.z, val.w};
 #pragma unroll
@@ -635,9 +674,25 @@ void quant_tile_kernel(QuantArgs p) {
   // PRO_SILU_BWD_PAIR: one workgroup produces the dgate tile and its dup twin (half / 128 column
   // tiles further right) from one read of grad_h, gate and up
   const int tiles_n_grid = PRO == PRO_SILU_BWD_PAIR ? p.tiles_n / 2 : p.tiles_n;
-  const int tc = (int)(bid % tiles_n_grid); bid /= tiles_n_grid;
-  const int tr = (int)(bid % p.tiles_m);
-  const int64_t g = bid / p.tiles_m;
+  int tc, tr;
+  int64_t g;
+  const int64_t remapped = (int64_t)(p.tiles_m & ~7) * tiles_n_grid;
+  if (AM == A_ROW && bid < remapped) {
+    // Row scales are [M, tiles_n] floats: the column tiles of one row block each write one float of
+    // the same 32-byte sectors.  Workgroup b runs on XCD b % 8, so with the column tile as the
+    // fastest index those writes meet in eight different L2s and leave as one sector write per
+    // float (8x their bytes; 12 % of this kernel's write traffic).  Here XCD x takes the row
+    // blocks x, x + 8, ... and all column tiles of a row block run back to back on it: their
+    // floats merge into whole lines in that L2.  (A_ROW launches have one group.)
+    const int64_t s = bid >> 3;
+    tc = (int)(s % tiles_n_grid);
+    tr = (int)(s / tiles_n_grid) * 8 + (int)(bid & 7);
+    g = 0;
+  } else {
+    tc = (int)(bid % tiles_n_grid); bid /= tiles_n_grid;
+    tr = (int)(bid % p.tiles_m);
+    g = bid / p.tiles_m;
+  }
   // The caller may size the tensors for the largest row count a routing can produce and tell the
   // real one through device memory (no host round trip): tiles past it have nothing to do.
   if (p.row_limit && (int64_t)tr * 128 >= *p.row_limit) return;
@@ -653,6 +708,7 @@ static int launch_quant(const QuantArgs& a, int dtype, int64_t G, hipStream_t st
   const int64_t blocks = (int64_t)a.tiles_m * a.tiles_n * G;
   if (blocks == 0) return PT_OK;
   PT_REQUIRE(blocks < (1ll << 31), "quant: grid too large (%lld tiles)", (long long)blocks);
+  PT_REQUIRE(AM != A_ROW || G == 1, "quant: row-scaled launches take one group");  // the kernel's tile order relies on it
   if (dtype == PT_BF16)
     hipLaunchKernelGGL((quant_tile_kernel<bf16_tag, AM, BMODE, BL, BS>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
   else if (dtype == PT_F32)
