@@ -739,7 +739,10 @@ def main():
         "data": "synthetic (seed 0: x~N(0,1) bf16, weights~N(0,0.02), grad~N(0,1), router logits~N(0,1) softmax top-k)",
         "config": {
             "workload": args.workload, "kind": kind, "hidden": H, "moe_intermediate": I, "experts": E,
-            "top_k": k, "tokens": T, "routed_rows": rows, "zipf_s": zipf,
+            "top_k": k, "tokens": T, "routed_rows": rows,
+            # rows of the grouped tensors: every expert's rows padded to a multiple of 128
+            "padded_rows": int((-(-torch.bincount(eidx.cpu(), minlength=E) // 128) * 128).sum()),
+            "zipf_s": zipf,
             **({"zipf_bias": "b_e = scale * (log p_e - mean(log p)), p_e ~ rank_e^-s, ranks from a seeded permutation; "
                              "scale raised in steps of 0.25 until an expert is empty and one exceeds 4x the mean",
                 "zipf_bias_scale": ZIPF_BIAS_SCALE.get(zipf)} if zipf is not None else {}),

@@ -138,6 +138,40 @@ struct st_f32 {
   static __device__ __forceinline__ float round(float v) { return v; }
 };
 
+// The same 8-wide accesses with the non-temporal cache policy (data that is touched once and is
+// larger than the caches); NT = false is the plain access, so kernels can take the policy as a
+// compile-time switch.
+typedef uint32_t nt_u4 __attribute__((ext_vector_type(4)));
+template <typename S, bool NT>
+__device__ __forceinline__ void load8_policy(const void* p, float* v) {
+  if constexpr (!NT) {
+    S::load8(p, v);
+  } else if constexpr (S::kBytes == 2) {
+    const nt_u4 q = __builtin_nontemporal_load(reinterpret_cast<const nt_u4*>(p));
+    S::load8(&q, v);
+  } else {
+    nt_u4 q[2];
+    q[0] = __builtin_nontemporal_load(reinterpret_cast<const nt_u4*>(p));
+    q[1] = __builtin_nontemporal_load(reinterpret_cast<const nt_u4*>(p) + 1);
+    S::load8(q, v);
+  }
+}
+template <typename S, bool NT>
+__device__ __forceinline__ void store8_policy(void* p, const float* v) {
+  if constexpr (!NT) {
+    S::store8(p, v);
+  } else if constexpr (S::kBytes == 2) {
+    nt_u4 q;
+    S::store8(&q, v);
+    __builtin_nontemporal_store(q, reinterpret_cast<nt_u4*>(p));
+  } else {
+    nt_u4 q[2];
+    S::store8(q, v);
+    __builtin_nontemporal_store(q[0], reinterpret_cast<nt_u4*>(p));
+    __builtin_nontemporal_store(q[1], reinterpret_cast<nt_u4*>(p) + 1);
+  }
+}
+
 // ---- FP8 scale rule ------------------------------------------------------------------------
 // scale = 2^ceil(log2(max(amax,1e-4) * fl32(1/448))), clamped to 2^-126; rcp by exponent flip.
 __device__ __forceinline__ float fp8_scale_from_amax(float amax, float& rcp) {

@@ -19,6 +19,19 @@
 #include <stdlib.h>
 #include <string.h>
 
+// Cache policy of the logits' accesses (1 = non-temporal loads, 2 = non-temporal stores; build
+// switch, make EXTRA=-DPT_CE_NT=<bits>): a [N, V] logits matrix is larger than every cache and each
+// pass touches an element once.  Both on: the in-place backward runs 10 % faster (4096 x 151 936
+// bf16: 478 -> 428 us), the forward is level; either one alone changes nothing.
+#ifndef PT_CE_NT
+#define PT_CE_NT 3
+#endif
+#if PT_CE_NT & 1
+#define PT_CE_LDS_LOAD_NT " nt"
+#else
+#define PT_CE_LDS_LOAD_NT ""
+#endif
+
 namespace pt {
 
 static constexpr int kCeThreads = 1024;
@@ -192,7 +205,7 @@ __device__ __forceinline__ void unpack8(const ce_v4i& w, float* v) {
 __device__ __forceinline__ void ce_load_to_lds(ce_v4i rsrc, uint32_t voff, uint32_t soff, uint32_t lds_off) {
   soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
   lds_off = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_off);
-  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff),
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen" PT_CE_LDS_LOAD_NT " lds" ::"v"(voff), "s"(rsrc), "s"(soff),
                "s"(lds_off)
                : "memory");
 }
@@ -256,7 +269,7 @@ __global__ __launch_bounds__(1024) void ce_fwd_onchip_kernel(CeArgs p) {
       ce_load_to_lds(rsrc_words, (uint32_t)(tid & 63) * 16u, c0 * 16u, lds_base + (c0 - kCeRegChunks * kCeThreads) * 16u);
   }
 #pragma unroll
-  for (int i = 0; i < kCeRegChunks; ++i) cache[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kCeThreads * 16, 0);
+  for (int i = 0; i < kCeRegChunks; ++i) cache[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, i * kCeThreads * 16, (PT_CE_NT & 1) ? 2 : 0);
 #pragma unroll
   for (int i = 0; i < kCeRegChunks; ++i)
     if ((uint32_t)i * kCeThreads + tid < p.chunks) absorb(cache[i]);
@@ -307,12 +320,13 @@ __global__ __launch_bounds__(1024) void ce_fwd_onchip_kernel(CeArgs p) {
   for (int i = 0; i < kCeRegChunks; ++i) {
     const uint32_t c = (uint32_t)i * kCeThreads + tid;
     // a chunk past the row's end computes on zeros and its store is dropped by the descriptor
-    __builtin_amdgcn_raw_buffer_store_b128(grad_of(cache[i], c), rsrc, voff, i * kCeThreads * 16, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(grad_of(cache[i], c), rsrc, voff, i * kCeThreads * 16, (PT_CE_NT & 2) ? 2 : 0);
     __builtin_amdgcn_sched_barrier(0);
   }
 #pragma unroll 1
   for (uint32_t c = kCeRegChunks * kCeThreads + tid; c < p.chunks; c += kCeThreads)
-    *(ce_v4i*)(x + (int64_t)c * 16) = grad_of(s_over[c - kCeRegChunks * kCeThreads], c);
+    if (PT_CE_NT & 2) __builtin_nontemporal_store(grad_of(s_over[c - kCeRegChunks * kCeThreads], c), (ce_v4i*)(x + (int64_t)c * 16));
+    else *(ce_v4i*)(x + (int64_t)c * 16) = grad_of(s_over[c - kCeRegChunks * kCeThreads], c);
 }
 
 __global__ __launch_bounds__(1024) void ce_finish_kernel(const float* loss_rows, int64_t N, const int64_t* n_non_ignore,
@@ -347,13 +361,26 @@ __global__ __launch_bounds__(256) void ce_scale_kernel(CeArgs p, uint32_t blocks
     float v[4][8];
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-      if (c0 + q * 256 < p.chunks) S::load8(x + (int64_t)(c0 + q * 256) * 8 * S::kBytes, v[q]);
+      if (c0 + q * 256 < p.chunks) {
+        if (S::kBytes == 2 && (PT_CE_NT & 1)) {
+          const ce_v4i w = __builtin_nontemporal_load((const ce_v4i*)(x + (int64_t)(c0 + q * 256) * 16));
+          S::load8(&w, v[q]);
+        } else {
+          S::load8(x + (int64_t)(c0 + q * 256) * 8 * S::kBytes, v[q]);
+        }
+      }
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       if (c0 + q * 256 < p.chunks) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[q][i] = v[q][i] * s;
-        S::store8(x + (int64_t)(c0 + q * 256) * 8 * S::kBytes, v[q]);
+        if (S::kBytes == 2 && (PT_CE_NT & 2)) {
+          ce_v4i w;
+          S::store8(&w, v[q]);
+          __builtin_nontemporal_store(w, (ce_v4i*)(x + (int64_t)(c0 + q * 256) * 16));
+        } else {
+          S::store8(x + (int64_t)(c0 + q * 256) * 8 * S::kBytes, v[q]);
+        }
       }
     }
   } else {
