@@ -186,6 +186,78 @@ class GemmTimer:
         # modules imported `_lib` (the module), so they see the patched attribute
         return self
 
+    def install_all(self):
+        """Second mode, used after the timed region only: events around every other entry point too,
+        collected in ``other`` as (name, start, end, args)."""
+        self.other = []
+        self.all_enabled = False
+        import torch
+
+        from pith_train_amd import _lib
+
+        inner = _lib.call
+        timer = self
+
+        def call(name, *args):
+            if timer.all_enabled and name not in GemmTimer.NAMES:
+                a = torch.cuda.Event(enable_timing=True)
+                b = torch.cuda.Event(enable_timing=True)
+                a.record()
+                inner(name, *args)
+                b.record()
+                timer.other.append((name, a, b, args))
+            else:
+                inner(name, *args)
+
+        _lib.call = call
+        return self
+
+    def in_step_report(self, steps, padded_rows, routed_rows):
+        """HBM-bound entry points as they ran inside the step (after the kernels before them, with
+        the caches in the state the step leaves them in): average duration of one call, and for
+        the quantisers the algorithmic bytes (bf16 2 B, FP8 1 B, one fp32 scale per 128 elements,
+        source rows of a gather counted once) over it.  Row counts above the padded row count are
+        buffer capacities; the kernels stop at the real count, which is what is priced."""
+        sc = 4.0 / 128
+
+        def nbytes(name, a):
+            rows = lambda m: min(int(m), padded_rows)  # noqa: E731
+            if name == "pt_quant_rowwise_colwise":
+                return rows(a[2]) * a[3] * (4 + 2 * sc)
+            if name == "pt_quant_rowwise_colwise_rows":
+                return (min(rows(a[2]), routed_rows) * 2 + rows(a[2]) * (2 + 2 * sc)) * a[3] + 4 * rows(a[2])
+            if name in ("pt_silu_mul_quant_rowwise_colwise", "pt_clamped_swiglu_quant_rowwise_colwise"):
+                return rows(a[1]) * a[2] * (4 + 2 + 2 * sc)
+            if name in ("pt_silu_mul_bwd_quant_rowwise_colwise", "pt_clamped_swiglu_bwd_quant_rowwise_colwise"):
+                return rows(a[4]) * a[5] * (2 + 4 + 2 * (2 + 2 * sc))
+            if name == "pt_quant_blockwise_transpose_batched":
+                return a[2] * a[3] * a[4] * (3 + (1 if a[9] else 0))
+            if name == "pt_quant_blockwise_transpose_batched_into":
+                return a[2] * a[3] * a[4] * (3 + (1 if a[11] else 0))
+            if name in ("pt_quant_rowwise_transpose", "pt_quant_rowwise_transpose_ld"):
+                return a[2] * a[3] * (4 + 2 * sc)
+            if name in ("pt_quant_rowwise_blockwise_transpose", "pt_quant_rowwise_blockwise_transpose_ld"):
+                return a[2] * a[3] * (4 + sc)
+            return None
+
+        agg = {}
+        for name, a, b, args in self.other:
+            d = agg.setdefault(name, [0.0, 0, 0.0])
+            d[0] += a.elapsed_time(b) * 1e3
+            d[1] += 1
+            nb = nbytes(name, args)
+            d[2] += nb if nb else 0.0
+        out = []
+        for name, (us, n, nb) in sorted(agg.items(), key=lambda kv: -kv[1][0]):
+            row = {"entry_point": name, "calls_per_step": n / max(steps, 1), "us_per_call": round(us / n, 1),
+                   "us_per_step": round(us / max(steps, 1), 1)}
+            if nb:
+                gbs = nb / us / 1e3
+                row.update({"algorithmic_MB_per_call": round(nb / n / 1e6, 1), "GB/s": round(gbs, 0),
+                            "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 3)})
+            out.append(row)
+        return out
+
     def summary(self):
         out = {}
         for name, a, b, _ in self.records:
@@ -712,6 +784,20 @@ def main():
                                    "note": "FP8 weight cache kept across steps (one quantisation per optimizer step, "
                                            "as FP8WeightCacheControl does); not the headline value"}
 
+    padded_rows = int((-(-torch.bincount(eidx.cpu(), minlength=E) // 128) * 128).sum())
+    if not args.no_kernel_report:
+        # the HBM-bound kernels where they run: a few more steps with events around every entry point
+        timer.install_all()
+        step()
+        torch.cuda.synchronize()
+        timer.all_enabled = True
+        n_extra = min(args.steps, 10)
+        for _ in range(n_extra):
+            step()
+        torch.cuda.synchronize()
+        timer.all_enabled = False
+        extra["hbm_kernels_in_step"] = timer.in_step_report(n_extra, padded_rows, rows)
+
     if args.calibrate_copy:
         cr, ch = 65536, 2048  # 65536 rows x 2048 bf16 = 256 MiB read + 256 MiB written (+ 512 KiB of indices)
         csrc = torch.randn((cr, ch), device="cuda").bfloat16()
@@ -741,7 +827,7 @@ def main():
             "workload": args.workload, "kind": kind, "hidden": H, "moe_intermediate": I, "experts": E,
             "top_k": k, "tokens": T, "routed_rows": rows,
             # rows of the grouped tensors: every expert's rows padded to a multiple of 128
-            "padded_rows": int((-(-torch.bincount(eidx.cpu(), minlength=E) // 128) * 128).sum()),
+            "padded_rows": padded_rows,
             "zipf_s": zipf,
             **({"zipf_bias": "b_e = scale * (log p_e - mean(log p)), p_e ~ rank_e^-s, ranks from a seeded permutation; "
                              "scale raised in steps of 0.25 until an expert is empty and one exceeds 4x the mean",

@@ -208,15 +208,37 @@ __global__ __launch_bounds__(256) void segment_sum_kernel(const char* x, const i
   const int64_t h0 = (int64_t)blockIdx.x * 128 + cc * 8;
   float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   if (vec) {
-    if (h0 < H)
-      for (int64_t r = start + rl; r < end; r += 16) {
-        const int64_t src = row_index ? (int64_t)row_index[r] : r;
-        if (src < 0 || src >= x_rows) continue;
-        float v[8];
-        S::load8(x + (src * H + h0) * S::kBytes, v);
+    // Eight rows of the thread in flight at a time, and the row indices of the next eight are
+    // requested before this batch's data is waited for (an index and the row it names are two
+    // dependent memory latencies otherwise).  The additions stay in row order, so the sum has the
+    // bits of a one-row-at-a-time loop.
+    constexpr int U = 8;
+    auto indices = [&](int64_t r, int64_t (&src)[U]) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] += v[j];
+      for (int u = 0; u < U; ++u) {
+        const int64_t ru = r + 16 * u;
+        src[u] = ru < end ? (row_index ? (int64_t)row_index[ru] : ru) : -1;
+        if (src[u] >= x_rows) src[u] = -1;
       }
+    };
+    if (h0 < H) {
+      int64_t src[U], nxt[U];
+      indices(start + rl, src);
+      for (int64_t r = start + rl; r < end; r += 16 * U) {
+        // (rows that do not exist read row 0 and are not added: no branch around a load)
+        float v[U][8];
+#pragma unroll
+        for (int u = 0; u < U; ++u) S::load8(x + ((src[u] >= 0 ? src[u] : 0) * H + h0) * S::kBytes, v[u]);
+        indices(r + 16 * U, nxt);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[j] = src[u] >= 0 ? acc[j] + v[u][j] : acc[j];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) src[u] = nxt[u];
+      }
+    }
   } else {
     for (int64_t r = start + rl; r < end; r += 16) {
       const int64_t src = row_index ? (int64_t)row_index[r] : r;
