@@ -360,6 +360,15 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
       const int64_t pitch = p.ldx * Loader<T>::kBytes;
 #pragma unroll
       for (int i = 0; i < 8; ++i) f.template load_row<AM == A_BLOCK>(i, base + i * pitch);
+    } else if (FULL) {
+      // Gathered rows of an interior tile: all eight loads are issued without a branch around any of
+      // them (a row that does not exist reads row 0 and is zeroed afterwards); with the test in
+      // front of each load the compiler waits for one row before it asks for the next.
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f.load_row(i, xb + ((src[i] >= 0 ? (int64_t)src[i] : 0) * p.ldx + col0) * Loader<T>::kBytes);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (src[i] < 0) f.zero_row(i);
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
