@@ -47,9 +47,13 @@ static inline int bits_for(int n) { int b = 0; while ((1 << b) < n) ++b; return 
 // ---------------------------------------------------------------------------------------------
 // group_rows: counts -> bases -> ranks
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void gr_hist_kernel(const int64_t* keys, int64_t m, int G, int32_t* counts /*[W][G]*/) {
+// Also marks every entry of src_of as "no row" (the rank kernel, three launches later, overwrites
+// the entries that name one).
+__global__ __launch_bounds__(256) void gr_hist_kernel(const int64_t* keys, int64_t m, int G, int32_t* counts /*[W][G]*/,
+                                                      int32_t* src_of, int64_t cap) {
   extern __shared__ int32_t s_hist[];  // [4][G]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < cap; i += (int64_t)gridDim.x * 256) src_of[i] = -1;
   int32_t* h = s_hist + wave * G;
   for (int g = lane; g < G; g += 64) h[g] = 0;
   __builtin_amdgcn_wave_barrier();
@@ -626,8 +630,11 @@ extern "C" int64_t pt_group_rows_workspace_bytes(int64_t m, int32_t num_groups) 
   return align_up(W * num_groups * 4, 256) + align_up((int64_t)num_groups * 4, 256);
 }
 
-// The five launches of the stable counting sort; `workspace` holds the [W][G] chunk counts and the
-// G group starts (pt_group_rows_workspace_bytes), every byte of which is written before it is read.
+// The four launches of the stable counting sort (chunk histograms, scan over the chunks, scan over
+// the groups, ranks); `workspace` holds the [W][G] chunk counts and the G group starts
+// (pt_group_rows_workspace_bytes), every byte of which is written before it is read.  (One kernel
+// for both scans, with the last workgroup to finish doing the second, measured slower: the
+// device-scope fences it needs write back and invalidate the XCD's L2, 8 us against a 4 us launch.)
 static int group_rows_launch(const int64_t* keys, int64_t m, int32_t G, int32_t alignment, int32_t* offs, int32_t* ks,
                              int64_t* reverse, int32_t* src_of, int64_t cap, void* workspace, hipStream_t s) {
   const int64_t W = cdiv(m, kWaveKeys);
@@ -635,8 +642,7 @@ static int group_rows_launch(const int64_t* keys, int64_t m, int32_t G, int32_t 
   int32_t* group_start = (int32_t*)((char*)workspace + align_up(W * G * 4, 256));
   const unsigned blocks = (unsigned)cdiv(W, 4);
   const size_t lds = (size_t)4 * G * sizeof(int32_t);
-  fill_i32_kernel<<<(unsigned)cdiv(cap, 256), 256, 0, s>>>(src_of, cap, -1);
-  gr_hist_kernel<<<blocks, 256, lds, s>>>(keys, m, G, counts);
+  gr_hist_kernel<<<blocks, 256, lds, s>>>(keys, m, G, counts, src_of, cap);
   gr_scan_chunks_kernel<<<(unsigned)cdiv(G, 4), 256, 0, s>>>(counts, W, G, group_start);
   gr_scan_groups_kernel<<<1, 1024, 0, s>>>(G, alignment, offs, ks, group_start);
   gr_rank_kernel<<<blocks, 256, lds, s>>>(keys, m, G, bits_for(G), counts, group_start, reverse, src_of, cap);
