@@ -80,17 +80,32 @@ __global__ __launch_bounds__(256) void moe_combine_ep_fwd_kernel(CombineArgs p) 
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-    for (int j = 0; j < n; ++j) {
-      const char* mp = p.moe + (int64_t)s_row[j] * p.ld_moe + cb;
-      float m[8];
-      if (p.vec) load8_policy<S, (PT_COMBINE_NT & 1) != 0>(mp, m);
-      else {
+    if (p.vec) {
+      // Up to eight rows are requested together (a row past the list reads the first one again and
+      // is not used); the accumulation walks them in list order as before.
+      for (int j0 = 0; j0 < n; j0 += 8) {
+        float m[8][8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) m[i] = i < nval ? S::load1(mp + i * S::kBytes) : 0.f;
+        for (int u = 0; u < 8; ++u)
+          load8_policy<S, (PT_COMBINE_NT & 1) != 0>(p.moe + (int64_t)s_row[j0 + u < n ? j0 + u : j0] * p.ld_moe + cb, m[u]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const bool ok = j0 + u < n;
+          const float wj = s_w[ok ? j0 + u : j0];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[i] = ok ? S::round(acc[i] + S::round(m[u][i] * wj)) : acc[i];
+        }
       }
-      const float wj = s_w[j];
+    } else {
+      for (int j = 0; j < n; ++j) {
+        const char* mp = p.moe + (int64_t)s_row[j] * p.ld_moe + cb;
+        const float wj = s_w[j];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = S::round(acc[i] + S::round(m[i] * wj));
+        for (int i = 0; i < 8; ++i) {
+          const float mi = i < nval ? S::load1(mp + i * S::kBytes) : 0.f;
+          acc[i] = S::round(acc[i] + S::round(mi * wj));
+        }
+      }
     }
     const char* rp = p.res + t * p.ld_res + cb;
     char* op = p.out + t * p.ld_out + cb;
@@ -133,17 +148,28 @@ __global__ __launch_bounds__(256) void moe_combine_fwd_kernel(CombineArgs p) {
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-    for (int j = 0; j < p.k; ++j) {
-      const char* mp = p.moe + (t * p.k + j) * p.ld_moe + cb;
-      float m[8];
-      if (p.vec) load8_policy<S, (PT_COMBINE_NT & 1) != 0>(mp, m);
-      else {
+    if (p.vec) {
+      // up to eight rows requested together; the sum still runs over j = 0, 1, ... in order
+      for (int j0 = 0; j0 < p.k; j0 += 8) {
+        float m[8][8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) m[i] = i < nval ? S::load1(mp + i * S::kBytes) : 0.f;
+        for (int u = 0; u < 8; ++u)
+          load8_policy<S, (PT_COMBINE_NT & 1) != 0>(p.moe + (t * p.k + (j0 + u < p.k ? j0 + u : j0)) * p.ld_moe + cb, m[u]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const bool ok = j0 + u < p.k;
+          const float wj = w[ok ? j0 + u : j0];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[i] = ok ? acc[i] + m[u][i] * wj : acc[i];
+        }
       }
-      const float wj = w[j];
+    } else {
+      for (int j = 0; j < p.k; ++j) {
+        const char* mp = p.moe + (t * p.k + j) * p.ld_moe + cb;
+        const float wj = w[j];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = acc[i] + m[i] * wj;
+        for (int i = 0; i < 8; ++i) acc[i] = acc[i] + (i < nval ? S::load1(mp + i * S::kBytes) : 0.f) * wj;
+      }
     }
     char* op = p.out + t * p.ld_out + cb;
     if (p.res == nullptr) {
@@ -187,30 +213,59 @@ __global__ __launch_bounds__(256) void moe_combine_bwd_kernel(CombineArgs p) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) g[i] = i < nval ? S::load1(gp + i * S::kBytes) : 0.f;
     }
+    if (p.vec) {
+      // The rows of eight slots are requested together (a slot without a row reads the gradient
+      // chunk again, memory that certainly exists, and neither stores nor accumulates).
 #pragma unroll
-    for (int j = 0; j < kMaxTopK; ++j) {
-      if (j < p.k) {
-        const int64_t row = p.slot_row ? (int64_t)p.slot_row[t * p.k + j] : t * p.k + j;
-        if (row < 0 || (p.slot_row && row >= p.rows)) continue;  // slot without a row: its weight gradient stays zero
-        const char* mp = p.moe + row * p.ld_moe + cb;
-        char* dp = p.dmoe + row * p.ld_dmoe + cb;
-        float m[8], d[8];
-        if (p.vec) load8_policy<S, (PT_COMBINE_NT & 1) != 0>(mp, m);
-        else {
+      for (int j0 = 0; j0 < kMaxTopK; j0 += 8) {
+        if (j0 < p.k) {
+          int64_t row[8];
+          float m[8][8];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) m[i] = i < nval ? S::load1(mp + i * S::kBytes) : 0.f;
+          for (int u = 0; u < 8; ++u) {
+            const int j = j0 + u;
+            int64_t r = -1;
+            if (j < p.k) r = p.slot_row ? (int64_t)p.slot_row[t * p.k + j] : t * p.k + j;
+            if (p.slot_row && r >= p.rows) r = -1;
+            row[u] = r;
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            load8_policy<S, (PT_COMBINE_NT & 1) != 0>(row[u] >= 0 ? p.moe + row[u] * p.ld_moe + cb : gp, m[u]);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const bool ok = row[u] >= 0;
+            const float wj = w[j0 + u < p.k ? j0 + u : 0];
+            float d[8];
+            float acc = part[j0 + u];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              d[i] = g[i] * wj;
+              acc = fmaf(g[i], m[u][i], acc);
+            }
+            part[j0 + u] = ok ? acc : part[j0 + u];
+            if (ok) store8_policy<S, (PT_COMBINE_NT & 2) != 0>(p.dmoe + row[u] * p.ld_dmoe + cb, d);
+          }
         }
-        const float wj = w[j];
-        float acc = part[j];
+      }
+    } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          d[i] = g[i] * wj;
-          acc = fmaf(g[i], m[i], acc);
+      for (int j = 0; j < kMaxTopK; ++j) {
+        if (j < p.k) {
+          const int64_t row = p.slot_row ? (int64_t)p.slot_row[t * p.k + j] : t * p.k + j;
+          if (row < 0 || (p.slot_row && row >= p.rows)) continue;  // slot without a row: its weight gradient stays zero
+          const char* mp = p.moe + row * p.ld_moe + cb;
+          char* dp = p.dmoe + row * p.ld_dmoe + cb;
+          const float wj = w[j];
+          float acc = part[j];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float mi = i < nval ? S::load1(mp + i * S::kBytes) : 0.f;
+            acc = fmaf(g[i], mi, acc);
+            if (i < nval) S::store1(dp + i * S::kBytes, g[i] * wj);
+          }
+          part[j] = acc;
         }
-        part[j] = acc;
-        if (p.vec) store8_policy<S, (PT_COMBINE_NT & 2) != 0>(dp, d);
-        else
-          for (int i = 0; i < nval; ++i) S::store1(dp + i * S::kBytes, d[i]);
       }
     }
   }

@@ -349,16 +349,17 @@ __global__ __launch_bounds__(256) void gb_sum_kernel(const char* go, int64_t ld_
         for (int e = 0; e < 8; ++e) acc[u][e] = 0.f;
       for (int q = 0; q < cnt; ++q) {
         const char* src = go + source(q) * ld_go_b;
+        // (a chunk past the end of the row reads the lane's first chunk again and is not added:
+        // no branch around a load, which would make the wave wait for one before asking for the next)
         float v[4][8];
 #pragma unroll
         for (int u = 0; u < 4; ++u)
-          if (h0 + u * 512 < H) load8_policy<S, (PT_PERMUTE_NT & 1) != 0>(src + (h0 + u * 512) * S::kBytes, v[u]);
+          load8_policy<S, (PT_PERMUTE_NT & 1) != 0>(src + (h0 + u * 512 < H ? h0 + u * 512 : h0) * S::kBytes, v[u]);
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-          if (h0 + u * 512 < H) {
+        for (int u = 0; u < 4; ++u) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[u][e] += v[u][e];
-          }
+          for (int e = 0; e < 8; ++e) acc[u][e] = h0 + u * 512 < H ? acc[u][e] + v[u][e] : acc[u][e];
+        }
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
