@@ -26,6 +26,10 @@
 #ifndef PT_QUANT_NT
 #define PT_QUANT_NT (1 + 4 + 32)
 #endif
+// rows of the paired SwiGLU-backward prologue whose loads are in flight at a time
+#ifndef PT_QUANT_PAIR_ROWS
+#define PT_QUANT_PAIR_ROWS 2
+#endif
 
 namespace pt {
 
@@ -236,11 +240,11 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
     // Two rows in flight: row i + 2 is addressed through a register that an empty assembly statement
     // ties to the packed results of row i.  Left alone, the compiler starts all eight rows at once
     // (24 loads and their unpacked values: the whole register file, one wave per SIMD).
-    uint32_t gate[2] = {0u, 0u};  // always zero
+    uint32_t gate[PT_QUANT_PAIR_ROWS] = {};  // always zero
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       if (FULL || (col_ok && row0 + i < p.M)) {
-        const int64_t r = row0 + i + gate[i & 1];
+        const int64_t r = row0 + i + gate[i % PT_QUANT_PAIR_ROWS];
         float d[8], g[8], u[8], dg[8], du[8];
         q_load8_pro(xb + (r * p.ldx + col0) * 2, d);
         const char* gp = (const char*)p.x2 + (r * p.ldx2 + col0) * 2;
@@ -254,7 +258,7 @@ __device__ __forceinline__ void quant_tile_body(const QuantArgs& p, float (*s_co
         f_up.w[i][2] = pack_bf16x2(du[4], du[5]); f_up.w[i][3] = pack_bf16x2(du[6], du[7]);
         f.fence_row(i);
         f_up.fence_row(i);
-        asm volatile("" : "+v"(gate[i & 1]) : "v"(f.w[i][3]), "v"(f_up.w[i][3]));
+        asm volatile("" : "+v"(gate[i % PT_QUANT_PAIR_ROWS]) : "v"(f.w[i][3]), "v"(f_up.w[i][3]));
       } else {
         f.zero_row(i);
         f_up.zero_row(i);
