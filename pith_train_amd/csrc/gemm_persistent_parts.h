@@ -49,12 +49,33 @@ __device__ __forceinline__ v4i make_rsrc(const void* base, uint32_t bytes) {
 
 // Direct-to-LDS buffer loads: address = base + voff (per lane) + soff (uniform); lane l's data lands
 // at lds_off + 16*l (dwordx4) or lds_off + 4*l (dword).  lds_off is a wave-uniform LDS byte address.
+// (PT_GEMM_LOAD_A_MOD / PT_GEMM_LOAD_B_MOD, measurement builds: cache-policy modifiers, e.g. " nt", of
+// the row-split kernel's a and b operand loads.)
+#ifndef PT_GEMM_LOAD_A_MOD
+#define PT_GEMM_LOAD_A_MOD ""
+#endif
+#ifndef PT_GEMM_LOAD_B_MOD
+#define PT_GEMM_LOAD_B_MOD ""
+#endif
 __device__ __forceinline__ void dma16(v4i rsrc, uint32_t voff, uint32_t soff, uint32_t lds_off) {
   soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);  // uniform by construction; pin them to SGPRs
   lds_off = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_off);
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(rsrc), "s"(soff),
                "s"(lds_off)
                : "memory");
+}
+template <int OPERAND>  // 0: a, 1: b
+__device__ __forceinline__ void dma16_op(v4i rsrc, uint32_t voff, uint32_t soff, uint32_t lds_off) {
+  soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);
+  lds_off = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_off);
+  if (OPERAND == 0)
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen" PT_GEMM_LOAD_A_MOD " lds" ::"v"(voff), "s"(rsrc),
+                 "s"(soff), "s"(lds_off)
+                 : "memory");
+  else
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen" PT_GEMM_LOAD_B_MOD " lds" ::"v"(voff), "s"(rsrc),
+                 "s"(soff), "s"(lds_off)
+                 : "memory");
 }
 __device__ __forceinline__ void dma4(v4i rsrc, uint32_t voff, uint32_t soff, uint32_t lds_off) {
   soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)soff);

@@ -224,7 +224,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
     if (PT_GEMM_ABLATE_LOADS == 1) { l_in = false; l_ok = false; }
     if (k < 2) {
       const int q = 16 * k + 8 * l_half + wave;
-      dma16(rs_a, (l_in && 8 * q < l_a_rows) ? va : kOob, l_soA + (uint32_t)(8 * q) * (uint32_t)p.lda, l_sA + q * 1024);
+      dma16_op<0>(rs_a, (l_in && 8 * q < l_a_rows) ? va : kOob, l_soA + (uint32_t)(8 * q) * (uint32_t)p.lda, l_sA + q * 1024);
     } else if (k < 4) {
       if constexpr (BT) {
         // reduction rows 64 half + 0..63: row quad Q covers rows 4Q..4Q+3.  Rows past the end of a
@@ -232,10 +232,10 @@ __global__ __launch_bounds__(WGM * WGN * 64, 1) void fp8_gemm_nt_rowsplit_kernel
         // descriptor's: the hardware returns zeros for them (its range check includes the scalar
         // offset), so no lane needs a check of its own.
         const int Q = 16 * l_half + 8 * (k - 2) + wave;
-        dma16(rs_b, l_ok ? vbt : kOob, l_soB + (uint32_t)(4 * Q) * (uint32_t)p.ldb, l_sA + BM * BK + Q * 1024);
+        dma16_op<1>(rs_b, l_ok ? vbt : kOob, l_soB + (uint32_t)(4 * Q) * (uint32_t)p.ldb, l_sA + BM * BK + Q * 1024);
       } else {
         const int q = 8 * (2 * (k - 2) + (wave >> 2)) + 4 * l_half + (wave & 3);
-        dma16(rs_b, l_in ? vb : kOob, l_soB + (uint32_t)(8 * q) * (uint32_t)p.ldb, l_sA + BM * BK + q * 1024);
+        dma16_op<1>(rs_b, l_in ? vb : kOob, l_soB + (uint32_t)(8 * q) * (uint32_t)p.ldb, l_sA + BM * BK + q * 1024);
       }
     } else {
       // scales go with the first half of a block; with the second the same instruction is issued
