@@ -687,20 +687,33 @@ void quant_tile_kernel(QuantArgs p) {
   // PRO_SILU_BWD_PAIR: one workgroup produces the dgate tile and its dup twin (half / 128 column
   // tiles further right) from one read of grad_h, gate and up
   const int tiles_n_grid = PRO == PRO_SILU_BWD_PAIR ? p.tiles_n / 2 : p.tiles_n;
+  // Row-scaled launches (one group): which XCD runs which tile decides whether the 4-byte scale
+  // writes merge into whole lines.  Row scales are [M, tiles_n] floats, so the column tiles of one
+  // row block write neighbouring floats; column scales in the [N, tiles_m] layout put the same
+  // column of neighbouring row blocks next to each other.  Workgroup b runs on XCD b % 8: with the
+  // column tile as the fastest index all of those writes would meet in eight different L2s and
+  // leave as one 32-byte sector per float (8x their bytes; 12 % of the kernel's write traffic).
+  // So XCD x takes octets of row blocks (octet o with o % 8 == x) and runs an octet's tiles back
+  // to back, the eight row blocks of a column tile first: both kinds of neighbours are written by
+  // one XCD within a few microseconds and merge in its L2.  Row blocks that do not fill eight
+  // octets are dealt singly (row block r to XCD r % 8, its column tiles back to back: the row
+  // scales still merge), the last tiles_m % 8 in plain order.
   int tc, tr;
-  int64_t g;
+  int64_t g = 0;
+  const int64_t per_oct = 8 * (int64_t)tiles_n_grid;
+  const int oct_rows = ((p.tiles_m >> 3) & ~7) * 8;  // row blocks in whole rounds of eight octets
+  const int64_t oct_region = (int64_t)oct_rows * tiles_n_grid;
   const int64_t remapped = (int64_t)(p.tiles_m & ~7) * tiles_n_grid;
-  if (AM == A_ROW && bid < remapped) {
-    // Row scales are [M, tiles_n] floats: the column tiles of one row block each write one float of
-    // the same 32-byte sectors.  Workgroup b runs on XCD b % 8, so with the column tile as the
-    // fastest index those writes meet in eight different L2s and leave as one sector write per
-    // float (8x their bytes; 12 % of this kernel's write traffic).  Here XCD x takes the row
-    // blocks x, x + 8, ... and all column tiles of a row block run back to back on it: their
-    // floats merge into whole lines in that L2.  (A_ROW launches have one group.)
+  if (AM == A_ROW && bid < oct_region) {
     const int64_t s = bid >> 3;
+    const int64_t o = (s / per_oct) * 8 + (bid & 7);
+    const int r = (int)(s % per_oct);
+    tc = r >> 3;
+    tr = (int)o * 8 + (r & 7);
+  } else if (AM == A_ROW && bid < remapped) {
+    const int64_t b2 = bid - oct_region, s = b2 >> 3;
     tc = (int)(s % tiles_n_grid);
-    tr = (int)(s / tiles_n_grid) * 8 + (int)(bid & 7);
-    g = 0;
+    tr = oct_rows + (int)(s / tiles_n_grid) * 8 + (int)(b2 & 7);
   } else {
     tc = (int)(bid % tiles_n_grid); bid /= tiles_n_grid;
     tr = (int)(bid % p.tiles_m);
