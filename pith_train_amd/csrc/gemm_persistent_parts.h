@@ -148,6 +148,19 @@ __device__ __forceinline__ void store_staged_bf16_lines(const v16f& a0, const v1
   // p = (row r | row r+1) of the lane's column; the even lane of a pair takes both low halves (row r,
   // columns c and c+1), the odd lane both high halves (row r+1): one byte permute of own and neighbour
   const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
+#ifdef PT_GEMM_ABLATE_STAGING
+  // measurement build: the stores carry raw accumulator bits, no conversion and no staging
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const v16f& a = hf ? a1 : a0;
+      v4i w = v4i{__float_as_int(a[8 * h]), __float_as_int(a[8 * h + 1]), __float_as_int(a[8 * h + 2]), __float_as_int(a[8 * h + 3])};
+      __builtin_amdgcn_raw_buffer_store_b128(w, out, voff[2 * hf + h], soff, AUX);
+      asm volatile("s_nop 4" ::"v"(w) : "memory");
+    }
+  return;
+#endif
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {  // tile rows 0-15, then 16-31
 #pragma unroll
