@@ -32,8 +32,8 @@ HBM_PEAK_GBS = 8000.0
 # of known size).  FETCH_SIZE counts what the L2 asks of the fabric, whether the memory-side cache
 # or HBM answers: where successive waves of tiles re-read operand panels that the 4 MiB L2 of an
 # XCD cannot keep (GPT-OSS: 2.5x the algorithmic bytes) most of the excess is served by that cache.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-30b-a3b-moe": 746e6, "dsv2-lite-moe": 477e6, "gpt-oss-20b-moe": 2807e6,
-                                 "qwen3-decoder-linears-32k": 916e6}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-30b-a3b-moe": 747e6, "dsv2-lite-moe": 477e6, "gpt-oss-20b-moe": 2831e6,
+                                 "qwen3-decoder-linears-32k": 923e6}
 
 WORKLOADS = {
     # name: (kind, hidden, intermediate, experts, top_k, tokens, zipf)
