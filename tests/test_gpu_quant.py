@@ -57,6 +57,28 @@ def test_rowwise_colwise(M, N, dtype):
     _eq(got_t[3], ref[3], "ch_scale")
 
 
+@pytest.mark.parametrize("M", [63 * 128, 64 * 128, 65 * 128, 72 * 128, 130 * 128 + 40])
+def test_row_scaled_kernels_cover_every_tile_under_each_tile_order(M):
+    """The row-scaled kernels hand their 128 x 128 tiles to workgroups in three orders, chosen by the
+    number of row blocks: octets of row blocks per XCD (from 64 row blocks on), single row blocks
+    per XCD (the next multiple of 8), plain order (the rest).  Row counts on either side of every
+    switch, one of them ragged, against the oracle bit for bit."""
+    D = _ops()
+    N = 392  # three full column tiles and a ragged one
+    x = _mk((M, N), M + 5)
+    ref = Q.fp8cast_rowwise_transpose(x)
+    got = D.fp8cast_rowwise_transpose(x.cuda())
+    for g, r, w in zip(got, ref, ("tok_fp8", "tok_scale", "t_fp8", "t_scale")):
+        _eq(g, r, w)
+    if M % 128 == 0:
+        ref = Q.fp8cast_rowwise_colwise(x)
+        got = D.fp8cast_rowwise_colwise_t(x.cuda())
+        _eq(got[0], ref[0], "tok_fp8")
+        _eq(got[1], ref[1], "tok_scale")
+        _eq(got[2], ref[2].view(torch.uint8).T.contiguous().view(torch.float8_e4m3fn), "ch_t_fp8")
+        _eq(got[3], ref[3], "ch_scale")
+
+
 def test_transposed_outputs_are_contiguous_as_in_the_reference():
     """The public quantisers return freshly allocated contiguous tensors whatever the token count
     (reference: operators/deepgemm_quantize.py:429-482,575-629); only the private form that the
